@@ -1,0 +1,175 @@
+/*
+ * torchft_amd.h - C ABI of the MI355X-native replica-sync library (libtorchft_amd.so).
+ *
+ * The reference (pytorch-labs/torchft) has no FFI on this path: its replica
+ * synchronisation is a handful of Python loops that call stock torch ops per
+ * parameter tensor.  Each entry point below replaces one such loop (cited as
+ * file:line under the reference tree) with one multi-tensor HIP launch.
+ *
+ * Conventions
+ *   - plain C, no torch types; every pointer named "device" is a borrowed
+ *     device pointer, everything else is host memory;
+ *   - return 0 on success, a negative tft_status on error; tft_last_error()
+ *     returns a thread-local message for the last failing call on this thread;
+ *   - the library never allocates device memory, never synchronises and keeps
+ *     no mutable global state: each call validates its arguments on the host
+ *     and enqueues exactly one kernel on the caller's hipStream_t (passed as
+ *     void*; NULL is the legacy default stream);
+ *   - re-entrant: may be called concurrently from the training thread, the
+ *     autograd thread (DDP comm hook) and the checkpoint thread.
+ *
+ * Multi-tensor tables
+ *   A launch walks a table of T tensors with C pointer columns.  The caller
+ *   builds three device arrays:
+ *     ptrs        [C][T]  void*     column-major: ptrs[c * T + t]
+ *     numel       [T]     uint64_t  elements (bytes for tft_mt_copy_bytes)
+ *     chunk_start [T+1]   uint32_t  exclusive prefix sum of
+ *                                   ceil(numel[t] / chunk_elems)
+ *   One workgroup processes one chunk of chunk_elems consecutive elements of one
+ *   tensor.  tft_mt_plan() computes chunk_start on the host.  Tensors must be
+ *   contiguous; columns of one tensor may alias each other only where a
+ *   function says so.  Any alignment is accepted: a tensor whose columns are
+ *   all 16-byte aligned takes the 128-bit path, others a scalar path.
+ *
+ * Arithmetic (fp32 unless noted; this is what "parity" means for this library)
+ *   - the N replica contributions are added sequentially in replica order
+ *     r = 0 .. N-1, starting from contribution 0;
+ *   - a replica whose bit in participate_mask is clear contributes +0.0 and is
+ *     not read;
+ *   - the sum is divided (IEEE divide, not reciprocal multiply) by
+ *     num_participants, which may differ from popcount(participate_mask);
+ *   - bf16 inputs are widened to fp32, accumulated and divided in fp32, and
+ *     rounded to nearest-even once on store.
+ */
+#ifndef TORCHFT_AMD_H_
+#define TORCHFT_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TFT_ABI_VERSION 1
+#define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
+#define TFT_MIN_CHUNK_ELEMS 1024u
+
+typedef enum tft_status {
+  TFT_OK = 0,
+  TFT_ERR_INVALID_ARGUMENT = -1,
+  TFT_ERR_UNSUPPORTED = -2,
+  TFT_ERR_LAUNCH = -3
+} tft_status;
+
+typedef enum tft_dtype { TFT_F32 = 0, TFT_BF16 = 1 } tft_dtype;
+
+/* Host struct describing one multi-tensor table (the arrays live on the device). */
+typedef struct tft_mt_table {
+  const void* ptrs;            /* device: void*[n_cols * n_tensors], column-major */
+  const uint64_t* numel;       /* device: [n_tensors] */
+  const uint32_t* chunk_start; /* device: [n_tensors + 1] */
+  uint32_t n_tensors;
+  uint32_t n_cols;
+  uint32_t chunk_elems;  /* multiple of TFT_MIN_CHUNK_ELEMS */
+  uint32_t total_chunks; /* == chunk_start[n_tensors] */
+} tft_mt_table;
+
+/* Outer optimizer hyper-parameters: torch.optim.SGD as the reference drives it
+ * (torchft/local_sgd.py:223; lr=0.7, momentum=0.9, nesterov=True at
+ * torchft/local_sgd_test.py:112-114). */
+typedef struct tft_sgd_params {
+  float lr;
+  float momentum;
+  float dampening;
+  float weight_decay;
+  int32_t nesterov;   /* 0 / 1 */
+  int32_t first_step; /* 1: momentum buffer does not exist yet: buf = grad (not read) */
+} tft_sgd_params;
+
+int tft_abi_version(void);
+const char* tft_last_error(void);
+
+/* Host-only: fills chunk_start[0 .. n_tensors] for the given element counts and
+ * returns the total chunk count (>= 0) or a negative tft_status. */
+int64_t tft_mt_plan(const uint64_t* numel, uint32_t n_tensors, uint32_t chunk_elems,
+                    uint32_t* chunk_start);
+
+/* Chunk size the kernels were tuned with (elements; bytes for dtype < 0). */
+uint32_t tft_default_chunk_elems(int dtype);
+
+/*
+ * Manager.allreduce arithmetic on one flat buffer
+ * (torchft/manager.py:267-268 zero if not participating, :274 allreduce SUM over
+ * replicas, :287 divide by num_participants) in one pass:
+ *   out[i] = (sum over r of (mask bit r ? replicas[r][i] : +0)) / num_participants
+ * `replicas` is a HOST array of n_replicas device pointers; `out` may alias any
+ * of them (in-place allreduce).  n_replicas may be 0 with mask 0 (out = 0).
+ */
+int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
+                   uint32_t participate_mask, uint32_t num_participants, uint64_t numel,
+                   int dtype, void* stream);
+
+/*
+ * Same arithmetic over a tensor table.  Columns: [out_0 .. out_{n_outs-1},
+ * replica_0 .. replica_{n_replicas-1}], n_outs in {1, 2}; every out column
+ * receives the same value and may alias a replica column.
+ *   - n_outs = 1: DDP gradient buckets addressed through their per-parameter
+ *     views, so flatten/unflatten cost nothing (torchft/ddp.py:65-71 plus the
+ *     torch Reducer's copy-in/copy-out);
+ *   - n_outs = 2: LocalSGD weight averaging with the backup refreshed in the
+ *     same pass (torchft/local_sgd.py:151-174, _average + _save_parameters).
+ */
+int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_replicas,
+                      uint32_t participate_mask, uint32_t num_participants, int dtype,
+                      void* stream);
+
+/*
+ * DiLoCo outer step, fully fused (torchft/local_sgd.py:205-225 with the commit
+ * decision already known to be true).  Columns: [p, b, buf, replica_0 ..].
+ * Per element:
+ *   g    = (sum_r (replica_r - b)) / num_participants      (subtract, then sum)
+ *   d    = weight_decay ? fma(b, weight_decay, g) : g
+ *   buf' = first_step ? d : fma(d, 1 - dampening, momentum * buf)
+ *   e    = nesterov ? fma(buf', momentum, d) : buf'    (momentum == 0: e = d, buf untouched)
+ *   p = b = fma(e, -lr, b)
+ * `p` may alias a replica column.  fp32 only.
+ */
+int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
+                            uint32_t participate_mask, uint32_t num_participants,
+                            const tft_sgd_params* sgd, void* stream);
+
+/*
+ * Two-phase form for callers that must consult should_commit() between the
+ * reduction and the update (torchft/local_sgd.py:212-219 then :221-225).
+ *
+ * Phase 1, columns [g, p, b, replica_0 ..]:
+ *   g = (sum_r (replica_r - b)) / num_participants;  if restore_p: p = b.
+ *   `p` may alias a replica column; it is written after all reads.
+ * Phase 2, columns [p, b, buf, g]: the SGD update above with g read from
+ *   memory and the parameter value taken from b (p was restored to b).
+ */
+int tft_mt_pseudograd_avg_f32(const tft_mt_table* table, uint32_t n_replicas,
+                              uint32_t participate_mask, uint32_t num_participants,
+                              int restore_p, void* stream);
+int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, void* stream);
+
+/*
+ * Byte-exact multi-tensor gather/scatter.  Columns: [dst, src]; numel counts
+ * BYTES.  One kernel serves every copy loop of the path: backup save/restore
+ * (torchft/local_sgd.py:121-131), bucket flatten/unflatten (torch Reducer under
+ * torchft/ddp.py:52-63) and checkpoint pack/unpack into one staging buffer
+ * (the torch.save / torch.load seats at torchft/checkpointing.py:164,203).
+ * dst and src of one tensor must not overlap.
+ */
+int tft_mt_copy_bytes(const tft_mt_table* table, void* stream);
+
+/* Benchmark hook: selects a launch variant for later calls FROM THIS THREAD
+ * (thread-local; 0 restores the tuned default).  bits 0-3: loads in flight per
+ * stream per lane (1, 2, 4, 8); bit 4: plain instead of non-temporal accesses;
+ * bits 8-23: grid cap in workgroups per CU (0 = one chunk per workgroup). */
+void tft_set_launch_variant(uint32_t variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHFT_AMD_H_ */

@@ -1,0 +1,254 @@
+"""GPU parity: every kernel, called through the C ABI, against the CPU checker.
+
+The kernels and the checker perform the same IEEE operations in the same order
+(sequential replica sum, true divide, the fused multiply-adds torch's
+add(alpha=) kernels use), so these comparisons are bit-exact, which is stricter
+than the rtol 1e-6 (fp32) / 1e-2 (bf16) bars the path is specified with.
+"""
+
+import itertools
+
+import pytest
+import torch
+
+from helpers import assert_bits_equal
+from oracle import replica_sync as O
+from torchft_amd import ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 3, 4, 5, 255, 1023, 1024, 1025, 4099, 32768, 32769, 65536 + 7, 200_003]
+
+
+def mask_to_list(mask, n):
+    return [bool((mask >> r) & 1) for r in range(n)]
+
+
+def draw(n, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(n, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_replicas,mask,nump", [
+    (1, 0b1, 1), (1, 0b1, 5), (1, 0b0, 5), (2, 0b11, 2), (3, 0b101, 2), (4, 0b1011, 3),
+    (4, 0b1111, 4), (8, 0xFF, 8), (8, 0b10110101, 2), (0, 0, 3),
+])
+def test_reduce_avg_flat(device, dtype, n_replicas, mask, nump):
+    for numel in SIZES:
+        reps = [draw(numel, dtype, 10 * r + numel % 7) for r in range(n_replicas)]
+        if n_replicas:
+            want = O.manager_allreduce_(reps, mask_to_list(mask, n_replicas), nump, torch.float32)
+        else:
+            want = torch.zeros(numel, dtype=dtype)
+        out = torch.full((numel,), 7.0, dtype=dtype, device=device)
+        ops.reduce_avg_(out, [r.to(device) for r in reps], mask, nump)
+        assert_bits_equal(out, want, f"numel={numel}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reduce_avg_in_place_and_misaligned(device, dtype):
+    # out aliases replica 1; all buffers start 1 element past a 16-byte boundary
+    numel = 70_001
+    reps = [draw(numel + 1, dtype, 50 + r) for r in range(3)]
+    want = O.manager_allreduce_([r[1:] for r in reps], [True, True, True], 3, torch.float32)
+    dev = [r.to(device) for r in reps]
+    out = dev[1][1:]
+    ops.reduce_avg_(out, [d[1:] for d in dev], 0b111, 3)
+    assert_bits_equal(out, want)
+    # the guard element in front is untouched
+    assert_bits_equal(dev[1][:1], reps[1][:1])
+    # mixed: only one operand misaligned
+    dev2 = [r.to(device) for r in reps]
+    out2 = torch.empty(numel, dtype=dtype, device=device)
+    ops.reduce_avg_(out2, [dev2[0][1:], dev2[1][:-1], dev2[2][1:]], 0b111, 3)
+    want2 = O.manager_allreduce_([reps[0][1:], reps[1][:-1], reps[2][1:]], [True] * 3, 3, torch.float32)
+    assert_bits_equal(out2, want2)
+
+
+def test_reference_known_answers(device):
+    # torchft/manager_test.py:520-543: 1.0 with 5 participants -> 0.2; healing -> 0.0
+    t = torch.tensor([1.0], device=device)
+    ops.reduce_avg_(t, [t], 0b1, 5)
+    torch.testing.assert_close(t.cpu(), torch.tensor([1.0 / 5]))
+    t = torch.tensor([1.0], device=device)
+    ops.reduce_avg_(t, [t], 0b0, 5)
+    torch.testing.assert_close(t.cpu(), torch.tensor([0.0]))
+    # torchft/process_group_test.py:185-203: [1] + [2] == [3]
+    a, b = torch.tensor([1.0], device=device), torch.tensor([2.0], device=device)
+    ops.reduce_avg_(a, [a, b], 0b11, 1)
+    torch.testing.assert_close(a.cpu(), torch.tensor([3.0]))
+
+
+def _mlp_workload(n_replicas, seed_shift=0):
+    shapes = workloads.mlp_shapes() + [("odd", (7, 3)), ("empty", (0,)), ("one", (1,))]
+    wl = workloads.make_diloco_workload(shapes, n_replicas, torch.device("cpu"))
+    return wl
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_outs", [1, 2])
+def test_mt_reduce_avg(device, dtype, n_outs):
+    wl = _mlp_workload(3)
+    reps = [[t.to(dtype) for t in rep] for rep in wl.replicas]
+    want = [
+        O.manager_allreduce_([rep[t] for rep in reps], [True, False, True], 2, torch.float32)
+        for t in range(len(wl.backup))
+    ]
+    dev = [[t.to(device) for t in rep] for rep in reps]
+    outs = [dev[0]] + ([[torch.empty_like(t) for t in dev[0]]] if n_outs == 2 else [])
+    ops.mt_reduce_avg(outs, dev, 0b101, 2)
+    for col in outs:
+        for got, w, name in zip(col, want, wl.names):
+            assert_bits_equal(got, w, name)
+    # replica 1 (not participating) was not written
+    for got, src in zip(dev[1], reps[1]):
+        assert_bits_equal(got, src)
+
+
+SGD_CASES = [
+    dict(lr=0.7, momentum=0.9, nesterov=True),
+    dict(lr=0.7, momentum=0.9, nesterov=False),
+    dict(lr=0.3, momentum=0.8, dampening=0.1, weight_decay=0.01),
+    dict(lr=0.5),
+    dict(lr=0.5, weight_decay=0.1),
+]
+
+
+@pytest.mark.parametrize("sgd_kw", SGD_CASES)
+@pytest.mark.parametrize("n_replicas,mask,nump", [(1, 1, 1), (2, 0b11, 2), (4, 0b1011, 3), (8, 0xFF, 8)])
+def test_diloco_fused_two_steps(device, sgd_kw, n_replicas, mask, nump):
+    """First step (no momentum state) then a steady-state step, against the checker."""
+    wl = _mlp_workload(n_replicas)
+    sgd = ops.OuterSGD(**sgd_kw)
+    kw = dict(lr=sgd.lr, momentum=sgd.momentum, dampening=sgd.dampening,
+              weight_decay=sgd.weight_decay, nesterov=sgd.nesterov)
+    part = mask_to_list(mask, n_replicas)
+    b_dev = [t.to(device) for t in wl.backup]
+    p_dev = [torch.empty_like(t) for t in b_dev]
+    m_dev = [torch.full_like(t, float("nan")) for t in b_dev] if sgd.momentum else None
+    backup, bufs = wl.backup, None
+    table = None
+    for step in range(2):
+        reps = [workloads.drifted_replica(backup, 1e-3, 77 + 10 * step + r) for r in range(n_replicas)]
+        want = O.diloco_perform_sync(reps, backup, bufs, part, nump, True, **kw)
+        reps_dev = [[t.to(device) for t in rep] for rep in reps]
+        ops.mt_diloco_outer(p_dev, b_dev, m_dev, reps_dev, sgd, step == 0, mask, nump)
+        for i, name in enumerate(wl.names):
+            assert_bits_equal(p_dev[i], want["params"][i], f"step {step} params {name}")
+            assert_bits_equal(b_dev[i], want["backup"][i], f"step {step} backup {name}")
+            if sgd.momentum:
+                assert_bits_equal(m_dev[i], want["momentum"][i], f"step {step} momentum {name}")
+        backup, bufs = want["backup"], (want["momentum"] if sgd.momentum else None)
+
+
+def test_diloco_two_phase_matches_fused_and_checker(device):
+    wl = _mlp_workload(2)
+    sgd = ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True)
+    bufs = workloads.normal_tensors([(n, tuple(t.shape)) for n, t in zip(wl.names, wl.backup)],
+                                    1e-3, 5, torch.device("cpu"))
+    want = O.diloco_perform_sync(wl.replicas, wl.backup, bufs, [True, True], 2, True,
+                                 lr=0.7, momentum=0.9, nesterov=True)
+    b = [t.to(device) for t in wl.backup]
+    m = [t.to(device) for t in bufs]
+    reps = [[t.to(device) for t in rep] for rep in wl.replicas]
+    p = reps[0]  # live params of "this" replica: in place
+    g = [torch.empty_like(t) for t in b]
+    ops.mt_pseudograd_avg(g, p, b, reps, restore_params=True)
+    for i, name in enumerate(wl.names):
+        assert_bits_equal(g[i], want["grads"][i], f"grad {name}")
+        assert_bits_equal(p[i], wl.backup[i], f"restored {name}")
+    ops.mt_outer_sgd(p, b, m, g, sgd, first_step=False)
+    for i, name in enumerate(wl.names):
+        assert_bits_equal(p[i], want["params"][i], f"params {name}")
+        assert_bits_equal(b[i], want["backup"][i], f"backup {name}")
+        assert_bits_equal(m[i], want["momentum"][i], f"momentum {name}")
+
+
+def test_diloco_no_commit_leaves_state(device):
+    """Phase 1 only (should_commit() false): params == backup, backup and momentum untouched."""
+    wl = _mlp_workload(2)
+    want = O.diloco_perform_sync(wl.replicas, wl.backup, None, [True, True], 2, False, lr=0.7,
+                                 momentum=0.9, nesterov=True)
+    b = [t.to(device) for t in wl.backup]
+    reps = [[t.to(device) for t in rep] for rep in wl.replicas]
+    g = [torch.empty_like(t) for t in b]
+    ops.mt_pseudograd_avg(g, reps[0], b, reps, restore_params=True)
+    for i, name in enumerate(wl.names):
+        assert_bits_equal(reps[0][i], want["params"][i], name)
+        assert_bits_equal(b[i], want["backup"][i], name)
+        assert_bits_equal(g[i], want["grads"][i], name)
+
+
+def test_localsgd_average_with_backup_refresh(device):
+    wl = _mlp_workload(2)
+    want = O.localsgd_perform_sync(wl.replicas, wl.backup, [True, True], 2, True)
+    reps = [[t.to(device) for t in rep] for rep in wl.replicas]
+    b = [t.to(device) for t in wl.backup]
+    ops.mt_reduce_avg([reps[0], b], reps)
+    for i, name in enumerate(wl.names):
+        assert_bits_equal(reps[0][i], want["params"][i], name)
+        assert_bits_equal(b[i], want["backup"][i], name)
+
+
+@pytest.mark.parametrize("src_off,dst_off", [(0, 0), (16, 32), (4, 8), (4, 0), (1, 1), (3, 6), (2, 2)])
+def test_mt_copy_bytes_alignments(device, src_off, dst_off):
+    sizes = [0, 1, 5, 16, 17, 4096, 262144, 262144 + 33, 1_000_003]
+    g = torch.Generator().manual_seed(3)
+    srcs_cpu = [torch.randint(0, 256, (n + src_off,), dtype=torch.uint8, generator=g) for n in sizes]
+    srcs = [t.to(device)[src_off:] for t in srcs_cpu]
+    dst_full = [torch.full((n + dst_off + 5,), 0xAB, dtype=torch.uint8, device=device) for n in sizes]
+    dsts = [t[dst_off:dst_off + n] for t, n in zip(dst_full, sizes)]
+    ops.mt_copy(dsts, srcs)
+    for full, src, n in zip(dst_full, srcs_cpu, sizes):
+        want = torch.full((n + dst_off + 5,), 0xAB, dtype=torch.uint8)
+        want[dst_off:dst_off + n] = src[src_off:]
+        assert_bits_equal(full, want, f"n={n}")
+
+
+def test_mt_copy_mixed_dtypes(device):
+    srcs_cpu = [torch.randn(1000).bfloat16(), torch.randn(333), torch.arange(7, dtype=torch.int64)]
+    srcs = [t.to(device) for t in srcs_cpu]
+    dsts = [torch.empty_like(t) for t in srcs]
+    ops.mt_copy(dsts, srcs)
+    for d, s in zip(dsts, srcs_cpu):
+        assert_bits_equal(d, s)
+
+
+def test_launch_variants_agree(device):
+    """Every tuning variant computes the same bits."""
+    wl = _mlp_workload(2)
+    sgd = ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True)
+    want = O.diloco_perform_sync(wl.replicas, wl.backup, None, [True, True], 2, True, lr=0.7,
+                                 momentum=0.9, nesterov=True)
+    try:
+        for unroll, plain, cap in itertools.product([1, 2, 4], [0, 1], [0, 2]):
+            ops.set_launch_variant(unroll | (plain << 4) | (cap << 8))
+            b = [t.to(device) for t in wl.backup]
+            m = [torch.empty_like(t) for t in b]
+            p = [torch.empty_like(t) for t in b]
+            reps = [[t.to(device) for t in rep] for rep in wl.replicas]
+            ops.mt_diloco_outer(p, b, m, reps, sgd, True)
+            for i, name in enumerate(wl.names):
+                assert_bits_equal(p[i], want["params"][i], f"variant {unroll}/{plain}/{cap} {name}")
+                assert_bits_equal(m[i], want["momentum"][i], f"variant {unroll}/{plain}/{cap} {name}")
+    finally:
+        ops.set_launch_variant(0)
+
+
+def test_argument_errors(device):
+    x = torch.zeros(8, device=device)
+    with pytest.raises(ValueError):
+        ops.reduce_avg_(x, [x] * 9)
+    with pytest.raises(ValueError):
+        ops.reduce_avg_(x, [x], 0b10, 1)
+    with pytest.raises(ValueError):
+        ops.reduce_avg_(x, [x], 0b1, 0)
+    with pytest.raises(ValueError):
+        ops.reduce_avg_(x, [torch.zeros(9, device=device)])
+    with pytest.raises(RuntimeError):
+        ops.reduce_avg_(torch.zeros(8), [torch.zeros(8)])
+    with pytest.raises(TypeError):
+        ops.reduce_avg_(x.double(), [x.double()])
+    with pytest.raises(ValueError):
+        ops.reduce_avg_(torch.zeros(4, 4, device=device).t(), [x[:16]])

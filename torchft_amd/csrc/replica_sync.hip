@@ -1,0 +1,706 @@
+// Replica-sync streaming kernels for MI355X (gfx950) and their C ABI.
+//
+// Every kernel here is HBM-bound elementwise work over a table of tensors: one
+// workgroup of 256 lanes (4 wavefronts of 64) owns one chunk of consecutive
+// elements of one tensor, finds its tensor by binary search over a small prefix
+// array (uniform across the workgroup, so it runs on the scalar unit), and
+// streams the chunk with 128-bit accesses, several independent loads in flight
+// per lane and per stream.  Nothing is reused, so accesses are non-temporal by
+// default to keep the L2 / Infinity Cache from being churned.  No LDS, no MFMA:
+// the arithmetic intensity is below 1 flop/byte.
+//
+// Entry points are declared and documented in include/torchft_amd.h.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "torchft_amd.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxCols = TFT_MAX_REPLICAS + 3;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+thread_local char g_err[512] = "";
+thread_local uint32_t g_variant = 0;
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// ---------------------------------------------------------------------------
+// Element types: how a 16-byte vector is widened to fp32 lanes and back.
+// ---------------------------------------------------------------------------
+struct F32 {
+  typedef float elem_t;
+  static constexpr int kVec = 4;
+  __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(raw[i]);
+  }
+  __device__ static inline u32x4 narrow(const float (&v)[kVec]) {
+    u32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = __float_as_uint(v[i]);
+    return raw;
+  }
+  __device__ static inline float widen1(float x) { return x; }
+  __device__ static inline float narrow1(float x) { return x; }
+};
+
+__device__ inline uint32_t f32_to_bf16_bits(float f) {
+  // round to nearest even; NaN collapses to the canonical quiet NaN (what
+  // c10::BFloat16 does on the host)
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+struct BF16 {
+  typedef uint16_t elem_t;
+  static constexpr int kVec = 8;
+  __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(raw[i] << 16);
+      v[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+    }
+  }
+  __device__ static inline u32x4 narrow(const float (&v)[kVec]) {
+    u32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      raw[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+    return raw;
+  }
+  __device__ static inline float widen1(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
+  __device__ static inline uint16_t narrow1(float x) { return (uint16_t)f32_to_bf16_bits(x); }
+};
+
+template <bool NT>
+__device__ inline u32x4 load16(const void* p) {
+  if (NT) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return *reinterpret_cast<const u32x4*>(p);
+}
+template <bool NT>
+__device__ inline void store16(void* p, const u32x4& v) {
+  if (NT)
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+  else
+    *reinterpret_cast<u32x4*>(p) = v;
+}
+
+// ---------------------------------------------------------------------------
+// Locators: map a chunk index to (column base pointers, element count).
+// ---------------------------------------------------------------------------
+struct TableArgs {
+  void* const* ptrs;
+  const uint64_t* numel;
+  const uint32_t* chunk_start;
+  uint32_t n_tensors;
+  uint32_t chunk_elems;
+  uint32_t total_chunks;
+};
+
+struct FlatArgs {  // one tensor, pointers carried in the kernel arguments
+  void* ptrs[kMaxCols];
+  uint64_t numel;
+  uint32_t chunk_elems;
+  uint32_t total_chunks;
+};
+
+template <int NCOL>
+struct TableLocator {
+  typedef TableArgs args_t;
+  __device__ static inline uint32_t locate(const TableArgs& a, uint32_t chunk, uint32_t cols,
+                                           char* (&ptr)[NCOL], size_t esize) {
+    // largest t with chunk_start[t] <= chunk
+    uint32_t lo = 0, hi = a.n_tensors;
+    while (hi - lo > 1) {
+      uint32_t mid = (lo + hi) >> 1;
+      if (a.chunk_start[mid] <= chunk)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    const uint64_t numel = a.numel[lo];
+    const uint64_t base = (uint64_t)(chunk - a.chunk_start[lo]) * a.chunk_elems;
+    const uint64_t left = numel - base;
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c)
+      ptr[c] = ((cols >> c) & 1u)
+                   ? static_cast<char*>(a.ptrs[(size_t)c * a.n_tensors + lo]) + base * esize
+                   : nullptr;
+    return left < a.chunk_elems ? (uint32_t)left : a.chunk_elems;
+  }
+};
+
+template <int NCOL>
+struct FlatLocator {
+  typedef FlatArgs args_t;
+  __device__ static inline uint32_t locate(const FlatArgs& a, uint32_t chunk, uint32_t cols,
+                                           char* (&ptr)[NCOL], size_t esize) {
+    const uint64_t base = (uint64_t)chunk * a.chunk_elems;
+    const uint64_t left = a.numel - base;
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c)
+      ptr[c] = ((cols >> c) & 1u) ? static_cast<char*>(a.ptrs[c]) + base * esize : nullptr;
+    return left < a.chunk_elems ? (uint32_t)left : a.chunk_elems;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// The streaming skeleton.  Op supplies:
+//   NCOL            number of pointer columns
+//   rmask()/wmask() which columns are loaded / stored (uniform)
+//   apply(v)        per-element arithmetic on v[NCOL] (fp32)
+// ---------------------------------------------------------------------------
+template <class E, class Op, int U, bool NT, bool CHECK>
+__device__ inline void stream_block(char* const (&ptr)[Op::NCOL], const Op& op, uint32_t v0,
+                                    uint32_t nvec, uint32_t rmask, uint32_t wmask) {
+  constexpr int NCOL = Op::NCOL;
+  constexpr int V = E::kVec;
+  u32x4 raw[NCOL][U];
+#pragma unroll
+  for (int c = 0; c < NCOL; ++c) {
+    if ((rmask >> c) & 1u) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * kThreads + threadIdx.x;
+        if (!CHECK || v < nvec)
+          raw[c][u] = load16<NT>(ptr[c] + (size_t)v * 16);
+        else
+          raw[c][u] = u32x4{0, 0, 0, 0};
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) raw[c][u] = u32x4{0, 0, 0, 0};
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float lanes[NCOL][V];
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c) E::widen(raw[c][u], lanes[c]);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      float v[NCOL];
+#pragma unroll
+      for (int c = 0; c < NCOL; ++c) v[c] = lanes[c][i];
+      op.apply(v);
+#pragma unroll
+      for (int c = 0; c < NCOL; ++c) lanes[c][i] = v[c];
+    }
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c) raw[c][u] = E::narrow(lanes[c]);
+  }
+#pragma unroll
+  for (int c = 0; c < NCOL; ++c) {
+    if ((wmask >> c) & 1u) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * kThreads + threadIdx.x;
+        if (!CHECK || v < nvec) store16<NT>(ptr[c] + (size_t)v * 16, raw[c][u]);
+      }
+    }
+  }
+}
+
+template <class E, class Op>
+__device__ inline void scalar_range(char* const (&ptr)[Op::NCOL], const Op& op, uint32_t begin,
+                                    uint32_t end, uint32_t rmask, uint32_t wmask) {
+  constexpr int NCOL = Op::NCOL;
+  typedef typename E::elem_t T;
+  for (uint32_t i = begin + threadIdx.x; i < end; i += kThreads) {
+    float v[NCOL];
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c)
+      v[c] = ((rmask >> c) & 1u) ? E::widen1(reinterpret_cast<const T*>(ptr[c])[i]) : 0.0f;
+    op.apply(v);
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c)
+      if ((wmask >> c) & 1u) reinterpret_cast<T*>(ptr[c])[i] = E::narrow1(v[c]);
+  }
+}
+
+template <class E, class Op, class Loc, int U, bool NT>
+__global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_t args, Op op) {
+  constexpr int NCOL = Op::NCOL;
+  constexpr int V = E::kVec;
+  const uint32_t rmask = op.rmask();
+  const uint32_t wmask = op.wmask();
+  for (uint32_t chunk = blockIdx.x; chunk < args.total_chunks; chunk += gridDim.x) {
+    char* ptr[NCOL];
+    const uint32_t n = Loc::locate(args, chunk, rmask | wmask, ptr, sizeof(typename E::elem_t));
+    uintptr_t bits = 0;
+#pragma unroll
+    for (int c = 0; c < NCOL; ++c) bits |= reinterpret_cast<uintptr_t>(ptr[c]);
+    if ((bits & 15u) == 0) {
+      const uint32_t nvec = n / V;
+      const uint32_t step = kThreads * U;
+      const uint32_t nfull = nvec - nvec % step;
+      uint32_t v0 = 0;
+      for (; v0 < nfull; v0 += step) stream_block<E, Op, U, NT, false>(ptr, op, v0, nvec, rmask, wmask);
+      if (v0 < nvec) stream_block<E, Op, U, NT, true>(ptr, op, v0, nvec, rmask, wmask);
+      if (nvec * V < n) scalar_range<E, Op>(ptr, op, nvec * V, n, rmask, wmask);
+    } else {
+      scalar_range<E, Op>(ptr, op, 0, n, rmask, wmask);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Ops.  Division and the two-rounding momentum update are spelled with the
+// round-to-nearest intrinsics so that the compiler cannot contract or
+// re-associate them; the fused multiply-adds are the ones torch's own add(alpha)
+// kernels perform.
+// ---------------------------------------------------------------------------
+template <int NREP>
+__device__ inline float replica_sum(const float* x, uint32_t mask) {
+  // sequential in replica order; a non-participant contributes +0
+  float s = (mask & 1u) ? x[0] : 0.0f;
+#pragma unroll
+  for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, ((mask >> r) & 1u) ? x[r] : 0.0f);
+  return s;
+}
+
+// columns: [out_0 .. out_{NOUT-1}, rep_0 .. rep_{NREP-1}]
+template <int NOUT, int NREP>
+struct ReduceAvgOp {
+  static constexpr int NCOL = NOUT + NREP;
+  uint32_t mask;  // participation bits
+  float n;        // num_participants
+  __device__ inline uint32_t rmask() const { return mask << NOUT; }
+  __device__ inline uint32_t wmask() const { return (1u << NOUT) - 1u; }
+  __device__ inline void apply(float (&v)[NCOL]) const {
+    float s = 0.0f;
+    if constexpr (NREP > 0) s = replica_sum<NREP>(&v[NOUT], mask);
+    s = __fdiv_rn(s, n);
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) v[o] = s;
+  }
+};
+
+struct SgdCoef {
+  float neg_lr, momentum, one_minus_dampening, weight_decay;
+  uint32_t nesterov, first_step;
+};
+
+__device__ inline float sgd_update(const SgdCoef& k, float g, float b, float& buf) {
+  float d = g;
+  if (k.weight_decay != 0.0f) d = __fmaf_rn(b, k.weight_decay, g);
+  float e = d;
+  if (k.momentum != 0.0f) {
+    float nb = d;
+    if (!k.first_step) nb = __fmaf_rn(d, k.one_minus_dampening, __fmul_rn(buf, k.momentum));
+    buf = nb;
+    e = k.nesterov ? __fmaf_rn(nb, k.momentum, d) : nb;
+  }
+  return __fmaf_rn(e, k.neg_lr, b);
+}
+
+template <int NREP>
+__device__ inline float pseudograd_avg(const float* x, float b, uint32_t mask, float n) {
+  // each replica subtracts the (shared) backup first, then the differences are summed
+  float s = (mask & 1u) ? __fsub_rn(x[0], b) : 0.0f;
+#pragma unroll
+  for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, ((mask >> r) & 1u) ? __fsub_rn(x[r], b) : 0.0f);
+  return __fdiv_rn(s, n);
+}
+
+// columns: [p, b, buf, rep_0 ..]
+template <int NREP>
+struct DilocoFusedOp {
+  static constexpr int NCOL = 3 + NREP;
+  uint32_t mask;
+  float n;
+  SgdCoef k;
+  __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
+  __device__ inline uint32_t rmask() const {
+    return (mask << 3) | 2u | ((uses_buf() && !k.first_step) ? 4u : 0u);
+  }
+  __device__ inline uint32_t wmask() const { return 3u | (uses_buf() ? 4u : 0u); }
+  __device__ inline void apply(float (&v)[NCOL]) const {
+    const float g = pseudograd_avg<NREP>(&v[3], v[1], mask, n);
+    const float p = sgd_update(k, g, v[1], v[2]);
+    v[0] = p;
+    v[1] = p;
+  }
+};
+
+// columns: [g, p, b, rep_0 ..]
+template <int NREP>
+struct PseudogradOp {
+  static constexpr int NCOL = 3 + NREP;
+  uint32_t mask;
+  float n;
+  uint32_t restore_p;
+  __device__ inline uint32_t rmask() const { return (mask << 3) | 4u; }
+  __device__ inline uint32_t wmask() const { return 1u | (restore_p ? 2u : 0u); }
+  __device__ inline void apply(float (&v)[NCOL]) const {
+    v[0] = pseudograd_avg<NREP>(&v[3], v[2], mask, n);
+    v[1] = v[2];
+  }
+};
+
+// columns: [p, b, buf, g]
+struct OuterSgdOp {
+  static constexpr int NCOL = 4;
+  SgdCoef k;
+  __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
+  __device__ inline uint32_t rmask() const {
+    return 8u | 2u | ((uses_buf() && !k.first_step) ? 4u : 0u);
+  }
+  __device__ inline uint32_t wmask() const { return 3u | (uses_buf() ? 4u : 0u); }
+  __device__ inline void apply(float (&v)[NCOL]) const {
+    const float p = sgd_update(k, v[3], v[1], v[2]);
+    v[0] = p;
+    v[1] = p;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Byte copy (gather / scatter).  columns: [dst, src]; numel counts bytes.
+// ---------------------------------------------------------------------------
+template <int U, bool NT>
+__global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {
+  for (uint32_t chunk = blockIdx.x; chunk < args.total_chunks; chunk += gridDim.x) {
+    char* ptr[2];
+    const uint32_t n = TableLocator<2>::locate(args, chunk, 3u, ptr, 1);
+    char* dst = ptr[0];
+    const char* src = ptr[1];
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+    uint32_t done = 0;
+    if ((bits & 15u) == 0) {
+      const uint32_t nvec = n / 16;
+      const uint32_t step = kThreads * U;
+      const uint32_t nfull = nvec - nvec % step;
+      uint32_t v0 = 0;
+      for (; v0 < nfull; v0 += step) {
+        u32x4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          raw[u] = load16<NT>(src + (size_t)(v0 + u * kThreads + threadIdx.x) * 16);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          store16<NT>(dst + (size_t)(v0 + u * kThreads + threadIdx.x) * 16, raw[u]);
+      }
+      for (uint32_t v = v0 + threadIdx.x; v < nvec; v += kThreads)
+        store16<NT>(dst + (size_t)v * 16, load16<NT>(src + (size_t)v * 16));
+      done = nvec * 16;
+    } else if ((bits & 3u) == 0) {
+      const uint32_t nw = n / 4;
+      for (uint32_t w = threadIdx.x; w < nw; w += kThreads)
+        reinterpret_cast<uint32_t*>(dst)[w] = reinterpret_cast<const uint32_t*>(src)[w];
+      done = nw * 4;
+    }
+    for (uint32_t i = done + threadIdx.x; i < n; i += kThreads) dst[i] = src[i];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side: validation and dispatch.
+// ---------------------------------------------------------------------------
+struct Variant {
+  int unroll;
+  bool nt;
+  uint32_t wg_per_cu;  // 0: one chunk per workgroup
+};
+
+Variant decode_variant(int default_unroll) {
+  Variant v{default_unroll, true, 0};
+  const uint32_t bits = g_variant;
+  if (bits & 0xfu) v.unroll = (int)(bits & 0xfu);
+  if (bits & 0x10u) v.nt = false;
+  v.wg_per_cu = (bits >> 8) & 0xffffu;
+  return v;
+}
+
+uint32_t grid_for(uint32_t total_chunks, const Variant& v) {
+  if (v.wg_per_cu == 0) return total_chunks;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess)
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const uint64_t cap = (uint64_t)cus * v.wg_per_cu;
+  return (uint32_t)(cap < total_chunks ? cap : total_chunks);
+}
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TFT_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return TFT_OK;
+}
+
+int check_table(const char* what, const tft_mt_table* t, uint32_t want_cols) {
+  if (!t) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: table is NULL", what);
+  if (t->n_cols != want_cols)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: table has %u columns, this call needs %u", what,
+                t->n_cols, want_cols);
+  if (t->chunk_elems < TFT_MIN_CHUNK_ELEMS || t->chunk_elems % TFT_MIN_CHUNK_ELEMS)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: chunk_elems %u is not a positive multiple of %u",
+                what, t->chunk_elems, TFT_MIN_CHUNK_ELEMS);
+  if (t->n_tensors == 0 || t->total_chunks == 0) return 1;  // nothing to do
+  if (!t->ptrs || !t->numel || !t->chunk_start)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: table arrays must not be NULL", what);
+  return TFT_OK;
+}
+
+int check_reduce(const char* what, uint32_t n_replicas, uint32_t mask, uint32_t num_participants) {
+  if (n_replicas > TFT_MAX_REPLICAS)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: %u replicas, at most %d per launch", what, n_replicas,
+                TFT_MAX_REPLICAS);
+  if (n_replicas < 32 && (mask >> n_replicas) != 0)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: participate_mask 0x%x names replicas >= %u", what,
+                mask, n_replicas);
+  if (num_participants == 0)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: num_participants must be >= 1", what);
+  return TFT_OK;
+}
+
+TableArgs table_args(const tft_mt_table* t) {
+  return TableArgs{static_cast<void* const*>(t->ptrs), t->numel, t->chunk_start,
+                   t->n_tensors, t->chunk_elems, t->total_chunks};
+}
+
+template <class E, class Op, class Loc>
+void launch_stream(const typename Loc::args_t& args, const Op& op, uint32_t total_chunks,
+                   int default_unroll, hipStream_t stream) {
+  const Variant v = decode_variant(default_unroll);
+  const dim3 grid(grid_for(total_chunks, v)), block(kThreads);
+#define TFT_LAUNCH(UU, NTT) \
+  hipLaunchKernelGGL((mt_stream_kernel<E, Op, Loc, UU, NTT>), grid, block, 0, stream, args, op)
+  if (v.nt) {
+    switch (v.unroll) {
+      case 1: TFT_LAUNCH(1, true); break;
+      case 2: TFT_LAUNCH(2, true); break;
+      default: TFT_LAUNCH(4, true); break;
+    }
+  } else {
+    switch (v.unroll) {
+      case 1: TFT_LAUNCH(1, false); break;
+      case 2: TFT_LAUNCH(2, false); break;
+      default: TFT_LAUNCH(4, false); break;
+    }
+  }
+#undef TFT_LAUNCH
+}
+
+// Expands `CALL(N)` for the run-time replica count.
+#define TFT_FOR_NREP(n, CALL) \
+  switch (n) {                \
+    case 0: CALL(0); break;   \
+    case 1: CALL(1); break;   \
+    case 2: CALL(2); break;   \
+    case 3: CALL(3); break;   \
+    case 4: CALL(4); break;   \
+    case 5: CALL(5); break;   \
+    case 6: CALL(6); break;   \
+    case 7: CALL(7); break;   \
+    default: CALL(8); break;  \
+  }
+
+SgdCoef make_coef(const tft_sgd_params* s) {
+  SgdCoef k;
+  k.neg_lr = -s->lr;
+  k.momentum = s->momentum;
+  k.one_minus_dampening = (float)(1.0 - (double)s->dampening);
+  k.weight_decay = s->weight_decay;
+  k.nesterov = s->nesterov ? 1u : 0u;
+  k.first_step = s->first_step ? 1u : 0u;
+  return k;
+}
+
+int check_sgd(const char* what, const tft_sgd_params* s) {
+  if (!s) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: sgd params are NULL", what);
+  if (s->nesterov && (s->momentum <= 0.0f || s->dampening != 0.0f))
+    return fail(TFT_ERR_INVALID_ARGUMENT,
+                "%s: nesterov needs momentum > 0 and dampening == 0 (got %g, %g)", what,
+                (double)s->momentum, (double)s->dampening);
+  return TFT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tft_abi_version(void) { return TFT_ABI_VERSION; }
+
+const char* tft_last_error(void) { return g_err; }
+
+void tft_set_launch_variant(uint32_t variant) { g_variant = variant; }
+
+uint32_t tft_default_chunk_elems(int dtype) {
+  if (dtype < 0) return 256u * 1024u;                  // bytes per copy chunk
+  return dtype == TFT_BF16 ? 64u * 1024u : 32u * 1024u;  // 128 KiB per stream either way
+}
+
+int64_t tft_mt_plan(const uint64_t* numel, uint32_t n_tensors, uint32_t chunk_elems,
+                    uint32_t* chunk_start) {
+  if (n_tensors && (!numel || !chunk_start))
+    return fail(TFT_ERR_INVALID_ARGUMENT, "tft_mt_plan: NULL array");
+  if (!chunk_start) return fail(TFT_ERR_INVALID_ARGUMENT, "tft_mt_plan: NULL chunk_start");
+  if (chunk_elems < TFT_MIN_CHUNK_ELEMS || chunk_elems % TFT_MIN_CHUNK_ELEMS)
+    return fail(TFT_ERR_INVALID_ARGUMENT,
+                "tft_mt_plan: chunk_elems %u is not a positive multiple of %u", chunk_elems,
+                TFT_MIN_CHUNK_ELEMS);
+  uint64_t total = 0;
+  for (uint32_t t = 0; t < n_tensors; ++t) {
+    chunk_start[t] = (uint32_t)total;
+    total += numel[t] / chunk_elems + (numel[t] % chunk_elems ? 1 : 0);
+    if (total > 0x7fffffffull)
+      return fail(TFT_ERR_UNSUPPORTED, "tft_mt_plan: more than 2^31 chunks; raise chunk_elems");
+  }
+  chunk_start[n_tensors] = (uint32_t)total;
+  return (int64_t)total;
+}
+
+int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
+                   uint32_t participate_mask, uint32_t num_participants, uint64_t numel,
+                   int dtype, void* stream) {
+  static const char* what = "tft_reduce_avg";
+  if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (dtype != TFT_F32 && dtype != TFT_BF16)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
+  if (numel == 0) return TFT_OK;
+  if (!out) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: out is NULL", what);
+  if (n_replicas && !replicas) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: replicas is NULL", what);
+  FlatArgs a{};
+  a.ptrs[0] = out;
+  for (uint32_t r = 0; r < n_replicas; ++r) {
+    if (((participate_mask >> r) & 1u) && !replicas[r])
+      return fail(TFT_ERR_INVALID_ARGUMENT, "%s: replica %u is NULL", what, r);
+    a.ptrs[1 + r] = const_cast<void*>(replicas[r]);
+  }
+  a.numel = numel;
+  a.chunk_elems = tft_default_chunk_elems(dtype);
+  const uint64_t chunks = (numel + a.chunk_elems - 1) / a.chunk_elems;
+  if (chunks > 0x7fffffffull) return fail(TFT_ERR_UNSUPPORTED, "%s: numel too large", what);
+  a.total_chunks = (uint32_t)chunks;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TFT_CALL(N)                                                                     \
+  do {                                                                                  \
+    ReduceAvgOp<1, N> op{participate_mask, (float)num_participants};                    \
+    if (dtype == TFT_F32)                                                               \
+      launch_stream<F32, ReduceAvgOp<1, N>, FlatLocator<1 + N>>(a, op, a.total_chunks, 4, s); \
+    else                                                                                \
+      launch_stream<BF16, ReduceAvgOp<1, N>, FlatLocator<1 + N>>(a, op, a.total_chunks, 2, s); \
+  } while (0)
+  TFT_FOR_NREP(n_replicas, TFT_CALL)
+#undef TFT_CALL
+  return check_launch(what);
+}
+
+int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_replicas,
+                      uint32_t participate_mask, uint32_t num_participants, int dtype,
+                      void* stream) {
+  static const char* what = "tft_mt_reduce_avg";
+  if (n_outs != 1 && n_outs != 2)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: n_outs must be 1 or 2, got %u", what, n_outs);
+  if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (dtype != TFT_F32 && dtype != TFT_BF16)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
+  if (int rc = check_table(what, table, n_outs + n_replicas)) return rc < 0 ? rc : TFT_OK;
+  const TableArgs a = table_args(table);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TFT_CALL2(O, N)                                                                   \
+  do {                                                                                    \
+    ReduceAvgOp<O, N> op{participate_mask, (float)num_participants};                      \
+    if (dtype == TFT_F32)                                                                 \
+      launch_stream<F32, ReduceAvgOp<O, N>, TableLocator<O + N>>(a, op, a.total_chunks, 4, s); \
+    else                                                                                  \
+      launch_stream<BF16, ReduceAvgOp<O, N>, TableLocator<O + N>>(a, op, a.total_chunks, 2, s); \
+  } while (0)
+#define TFT_CALL_O1(N) TFT_CALL2(1, N)
+#define TFT_CALL_O2(N) TFT_CALL2(2, N)
+  if (n_outs == 1) {
+    TFT_FOR_NREP(n_replicas, TFT_CALL_O1)
+  } else {
+    TFT_FOR_NREP(n_replicas, TFT_CALL_O2)
+  }
+#undef TFT_CALL_O1
+#undef TFT_CALL_O2
+#undef TFT_CALL2
+  return check_launch(what);
+}
+
+int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
+                            uint32_t participate_mask, uint32_t num_participants,
+                            const tft_sgd_params* sgd, void* stream) {
+  static const char* what = "tft_mt_diloco_outer_f32";
+  if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (int rc = check_sgd(what, sgd)) return rc;
+  if (int rc = check_table(what, table, 3 + n_replicas)) return rc < 0 ? rc : TFT_OK;
+  const TableArgs a = table_args(table);
+  const SgdCoef k = make_coef(sgd);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TFT_CALL(N)                                                                       \
+  do {                                                                                    \
+    DilocoFusedOp<N> op{participate_mask, (float)num_participants, k};                    \
+    launch_stream<F32, DilocoFusedOp<N>, TableLocator<3 + N>>(a, op, a.total_chunks, 2, s); \
+  } while (0)
+  TFT_FOR_NREP(n_replicas, TFT_CALL)
+#undef TFT_CALL
+  return check_launch(what);
+}
+
+int tft_mt_pseudograd_avg_f32(const tft_mt_table* table, uint32_t n_replicas,
+                              uint32_t participate_mask, uint32_t num_participants,
+                              int restore_p, void* stream) {
+  static const char* what = "tft_mt_pseudograd_avg_f32";
+  if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (int rc = check_table(what, table, 3 + n_replicas)) return rc < 0 ? rc : TFT_OK;
+  const TableArgs a = table_args(table);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TFT_CALL(N)                                                                      \
+  do {                                                                                   \
+    PseudogradOp<N> op{participate_mask, (float)num_participants, restore_p ? 1u : 0u};  \
+    launch_stream<F32, PseudogradOp<N>, TableLocator<3 + N>>(a, op, a.total_chunks, 2, s); \
+  } while (0)
+  TFT_FOR_NREP(n_replicas, TFT_CALL)
+#undef TFT_CALL
+  return check_launch(what);
+}
+
+int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, void* stream) {
+  static const char* what = "tft_mt_outer_sgd_f32";
+  if (int rc = check_sgd(what, sgd)) return rc;
+  if (int rc = check_table(what, table, 4)) return rc < 0 ? rc : TFT_OK;
+  const TableArgs a = table_args(table);
+  OuterSgdOp op{make_coef(sgd)};
+  launch_stream<F32, OuterSgdOp, TableLocator<4>>(a, op, a.total_chunks, 4,
+                                                  static_cast<hipStream_t>(stream));
+  return check_launch(what);
+}
+
+int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
+  static const char* what = "tft_mt_copy_bytes";
+  if (int rc = check_table(what, table, 2)) return rc < 0 ? rc : TFT_OK;
+  const TableArgs a = table_args(table);
+  const Variant v = decode_variant(4);
+  const dim3 grid(grid_for(a.total_chunks, v)), block(kThreads);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (v.nt) {
+    if (v.unroll >= 4)
+      hipLaunchKernelGGL((mt_copy_kernel<4, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((mt_copy_kernel<2, true>), grid, block, 0, s, a);
+  } else {
+    if (v.unroll >= 4)
+      hipLaunchKernelGGL((mt_copy_kernel<4, false>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((mt_copy_kernel<2, false>), grid, block, 0, s, a);
+  }
+  return check_launch(what);
+}
+
+}  // extern "C"
