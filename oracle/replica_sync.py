@@ -352,3 +352,61 @@ def c_diloco_outer(
         ctypes.c_uint64(p.numel()),
     )
     return p, b, m
+
+
+# ---------------------------------------------------------------------------
+# The reference loop as a timed CPU baseline
+# ---------------------------------------------------------------------------
+
+
+def make_gloo_world1():
+    """A ``ProcessGroupGloo`` of world size 1 over an in-process store: the backend the
+    reference's own tests run this path on (torchft/process_group.py:303-317)."""
+    import datetime
+
+    import torch.distributed as dist
+
+    store = dist.HashStore()
+    return dist.ProcessGroupGloo(store, 0, 1, datetime.timedelta(seconds=60))
+
+
+def diloco_reference_loop_(
+    pg,
+    params: Sequence[torch.Tensor],
+    backup: Sequence[torch.Tensor],
+    peers: Sequence[Sequence[torch.Tensor]],
+    outer_optimizer: torch.optim.Optimizer,
+    num_participants: int,
+) -> None:
+    """One committed DiLoCo sync written as the reference writes it: five per-tensor
+    loops of stock torch ops (torchft/local_sgd.py:205-239, torchft/manager.py:274-287),
+    in place on ``params`` / ``backup``; ``outer_optimizer`` must own ``params``.
+
+    ``pg`` is a world-size-1 process group (its all-reduce is the identity on this
+    replica's tensor); the other replicas of the job are the parameter lists in
+    ``peers``, whose pseudo-gradients are added in order, as a ring step would.
+    """
+    import torch.distributed as dist
+
+    # local_sgd.py:212-215
+    for p, b in zip(params, backup):
+        p.grad = p.data - b
+    # local_sgd.py:227-239 -> manager.py:274, 287
+    works = []
+    for t, p in enumerate(params):
+        for peer in peers:
+            p.grad.add_(peer[t] - backup[t])
+        opts = dist.AllreduceOptions()
+        opts.reduceOp = dist.ReduceOp.SUM
+        works.append(pg.allreduce([p.grad], opts))
+    for p, w in zip(params, works):
+        w.wait()
+        p.grad /= num_participants
+    # local_sgd.py:219
+    for p, b in zip(params, backup):
+        p.data.copy_(b)
+    # local_sgd.py:221-225
+    outer_optimizer.step()
+    for p, b in zip(params, backup):
+        b.copy_(p.data)
+    outer_optimizer.zero_grad()

@@ -646,7 +646,7 @@ int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
 #define TFT_CALL(N)                                                                       \
   do {                                                                                    \
     DilocoFusedOp<N> op{participate_mask, (float)num_participants, k};                    \
-    launch_stream<F32, DilocoFusedOp<N>, TableLocator<3 + N>>(a, op, a.total_chunks, 2, s); \
+    launch_stream<F32, DilocoFusedOp<N>, TableLocator<3 + N>>(a, op, a.total_chunks, 4, s); \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
