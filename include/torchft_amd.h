@@ -20,13 +20,16 @@
  *
  * Multi-tensor tables
  *   A launch walks a table of T tensors with C pointer columns.  The caller
- *   builds three device arrays:
+ *   builds four device arrays:
  *     ptrs        [C][T]  void*     column-major: ptrs[c * T + t]
  *     numel       [T]     uint64_t  elements (bytes for tft_mt_copy_bytes)
  *     chunk_start [T+1]   uint32_t  exclusive prefix sum of
  *                                   ceil(numel[t] / chunk_elems)
- *   One workgroup processes one chunk of chunk_elems consecutive elements of one
- *   tensor.  tft_mt_plan() computes chunk_start on the host.  Tensors must be
+ *     chunk_tensor[K]     uint32_t  tensor index of every chunk,
+ *                                   K = chunk_start[T]
+ *   A chunk is chunk_elems consecutive elements of one tensor; the kernels cut
+ *   it further into slabs of one 128-bit access per lane, one workgroup each.
+ *   tft_mt_plan() computes both arrays on the host.  Tensors must be
  *   contiguous; columns of one tensor may alias each other only where a
  *   function says so.  Any alignment is accepted: a tensor whose columns are
  *   all 16-byte aligned takes the 128-bit path, others a scalar path.
@@ -50,9 +53,9 @@
 extern "C" {
 #endif
 
-#define TFT_ABI_VERSION 1
+#define TFT_ABI_VERSION 2
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
-#define TFT_MIN_CHUNK_ELEMS 1024u
+#define TFT_MIN_CHUNK_ELEMS 8192u
 
 typedef enum tft_status {
   TFT_OK = 0,
@@ -68,9 +71,10 @@ typedef struct tft_mt_table {
   const void* ptrs;            /* device: void*[n_cols * n_tensors], column-major */
   const uint64_t* numel;       /* device: [n_tensors] */
   const uint32_t* chunk_start; /* device: [n_tensors + 1] */
+  const uint32_t* chunk_tensor; /* device: [total_chunks] */
   uint32_t n_tensors;
   uint32_t n_cols;
-  uint32_t chunk_elems;  /* multiple of TFT_MIN_CHUNK_ELEMS */
+  uint32_t chunk_elems;  /* power of two >= TFT_MIN_CHUNK_ELEMS */
   uint32_t total_chunks; /* == chunk_start[n_tensors] */
 } tft_mt_table;
 
@@ -89,10 +93,12 @@ typedef struct tft_sgd_params {
 int tft_abi_version(void);
 const char* tft_last_error(void);
 
-/* Host-only: fills chunk_start[0 .. n_tensors] for the given element counts and
- * returns the total chunk count (>= 0) or a negative tft_status. */
+/* Host-only: fills chunk_start[0 .. n_tensors] and, unless it is NULL,
+ * chunk_tensor[0 .. total) for the given element counts; returns the total chunk
+ * count (>= 0) or a negative tft_status.  Call once with chunk_tensor == NULL to
+ * size that array. */
 int64_t tft_mt_plan(const uint64_t* numel, uint32_t n_tensors, uint32_t chunk_elems,
-                    uint32_t* chunk_start);
+                    uint32_t* chunk_start, uint32_t* chunk_tensor);
 
 /* Chunk size the kernels were tuned with (elements; bytes for dtype < 0). */
 uint32_t tft_default_chunk_elems(int dtype);
@@ -164,9 +170,9 @@ int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, v
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream);
 
 /* Benchmark hook: selects a launch variant for later calls FROM THIS THREAD
- * (thread-local; 0 restores the tuned default).  bits 0-3: loads in flight per
- * stream per lane (1, 2, 4, 8); bit 4: plain instead of non-temporal accesses;
- * bits 8-23: grid cap in workgroups per CU (0 = one chunk per workgroup). */
+ * (thread-local; 0 restores the tuned default).  bits 0-3: 128-bit accesses per
+ * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; default 2);
+ * bit 4: plain instead of non-temporal accesses. */
 void tft_set_launch_variant(uint32_t variant);
 
 #ifdef __cplusplus

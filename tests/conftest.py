@@ -25,3 +25,20 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def device():
     return torch.device("cuda", 0)
+
+
+@pytest.fixture
+def cpu_ops(monkeypatch):
+    """Replaces the kernel wrappers by the CPU stand-in of tests/fake_backend.py and lets
+    device-placement checks accept CPU tensors, so host logic runs without a GPU."""
+    import fake_backend
+    from torchft_amd import local_sgd, ops
+
+    for name in fake_backend.PATCHED:
+        monkeypatch.setattr(ops, name, getattr(fake_backend, name))
+    monkeypatch.setattr(
+        local_sgd.LocalSGD, "_on_device", staticmethod(lambda params, backups: bool(params))
+    )
+    fake_backend.calls.clear()
+    return fake_backend
+

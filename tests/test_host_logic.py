@@ -1,0 +1,680 @@
+"""Host logic without a GPU: the reference's own unit tests for this path, re-expressed
+against torchft_amd's classes (torchft/local_sgd_test.py, ddp_test.py, optim_test.py,
+checkpointing_test.py and the allreduce / participation tests of manager_test.py).
+
+Where arithmetic is involved the ``cpu_ops`` fixture substitutes the kernels by the CPU
+checker, so what is tested here is control flow: call counts, the commit gate, rollback,
+error latching, optimizer-state handling, bucket bookkeeping.
+"""
+
+import threading
+import urllib.error
+from datetime import timedelta
+from typing import Dict
+from unittest.mock import MagicMock, create_autospec
+
+import pytest
+import torch
+from torch import nn, optim
+from torch.futures import Future
+
+from helpers import assert_bits_equal
+from oracle import replica_sync as O
+from torchft_amd import (
+    CheckpointServer,
+    DiLoCo,
+    DistributedDataParallel,
+    LocalSGD,
+    Manager,
+    OptimizerWrapper,
+    ProcessGroup,
+    ProcessGroupDummy,
+    ProcessGroupLocalReplicas,
+    PureDistributedDataParallel,
+    QuorumResult,
+    StaticQuorum,
+    WorldSizeMode,
+    workloads,
+)
+from torchft_amd.checkpointing import _timed_acquire
+from torchft_amd.ddp import compute_bucket_assignment
+from torchft_amd.manager import QuorumClient
+from torchft_amd.process_group import _DummyWork
+
+
+class SimpleModel(nn.Module):
+    def __init__(self) -> None:
+        super().__init__()
+        self.model = nn.Sequential(nn.Linear(3, 4), nn.ReLU(), nn.Linear(4, 5), nn.Sigmoid())
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.model(x)
+
+
+def _params_dict(m: nn.Module) -> Dict[str, torch.Tensor]:
+    return {name: p.data for name, p in m.named_parameters()}
+
+
+def _train_step(model, optimizer):
+    loss = model(torch.rand(2, 3)).mean()
+    loss.backward()
+    optimizer.step()
+
+
+# ---------------------------------------------------------------------------
+# torchft/local_sgd_test.py
+# ---------------------------------------------------------------------------
+
+def test_local_sgd_healthy():
+    model = SimpleModel()
+    optimizer = optim.SGD(model.parameters())
+    manager = create_autospec(Manager)
+    with LocalSGD(manager, model, optimizer, sync_every=2) as local_sgd:
+        assert local_sgd._local_step == 0
+        torch.testing.assert_close(local_sgd._backup_parameters, _params_dict(model))
+        _train_step(model, optimizer)
+        assert local_sgd._local_step == 1
+        assert manager.start_quorum.call_count == 0
+        _train_step(model, optimizer)
+        assert manager.start_quorum.call_count == 1
+        manager.should_commit.return_value = True
+        assert local_sgd._local_step == 0
+        torch.testing.assert_close(local_sgd._backup_parameters, _params_dict(model))
+        assert manager.should_commit.call_count == 1
+        assert manager.allreduce.call_count == 4
+
+
+def test_local_sgd_recovery():
+    model = SimpleModel()
+    optimizer = optim.SGD(model.parameters())
+    manager = create_autospec(Manager)
+    with LocalSGD(manager, model, optimizer, sync_every=2) as local_sgd:
+        torch.testing.assert_close(local_sgd._backup_parameters, _params_dict(model))
+        og = {k: v.clone() for k, v in model.state_dict().items()}
+        _train_step(model, optimizer)
+        for name, param in model.state_dict().items():
+            assert not torch.equal(og[name], param), f"Parameter {name} did not change."
+        assert local_sgd._local_step == 1
+        local_sgd._restore_parameters()
+        torch.testing.assert_close(local_sgd._backup_parameters, _params_dict(model))
+        torch.testing.assert_close(dict(model.state_dict()), og)
+
+
+def test_local_sgd_no_commit_and_exception_roll_back():
+    model = SimpleModel()
+    optimizer = optim.SGD(model.parameters())
+    manager = create_autospec(Manager)
+    manager.should_commit.return_value = False
+    og = {k: v.clone() for k, v in model.state_dict().items()}
+    with LocalSGD(manager, model, optimizer, sync_every=1):
+        _train_step(model, optimizer)  # sync happens, commit refused
+        torch.testing.assert_close(dict(model.state_dict()), og)
+    with pytest.raises(RuntimeError, match="boom"):
+        with LocalSGD(manager, model, optimizer, sync_every=5):
+            _train_step(model, optimizer)
+            raise RuntimeError("boom")
+    torch.testing.assert_close(dict(model.state_dict()), og)  # torchft/local_sgd.py:111-113
+    assert len(optimizer._optimizer_step_post_hooks) == 0  # hooks removed on exit
+
+
+def test_diloco_healthy(cpu_ops):
+    model = SimpleModel()
+    inner = optim.AdamW(model.parameters(), lr=4e-4, weight_decay=0.1, betas=(0.9, 0.95))
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = False
+    with DiLoCo(manager, model, inner, outer, sync_every=2) as diloco:
+        parameter_count = len(list(model.parameters()))
+        assert outer.state_dict()["state"] == {}
+        assert diloco._local_step == 0
+        torch.testing.assert_close(diloco._backup_parameters, _params_dict(model))
+        _train_step(model, inner)
+        assert diloco._local_step == 1
+        assert manager.start_quorum.call_count == 0
+        _train_step(model, inner)
+        assert manager.start_quorum.call_count == 1
+        manager.should_commit.return_value = True
+        assert diloco._local_step == 0
+        torch.testing.assert_close(diloco._backup_parameters, _params_dict(model))
+        assert manager.should_commit.call_count == 1
+        assert manager.allreduce.call_count == parameter_count
+        assert len(outer.state_dict()["state"]) == parameter_count
+        assert all(p.grad is None for p in model.parameters())
+
+
+def test_diloco_requires_sync_quorum():
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = True
+    model = SimpleModel()
+    with pytest.raises(ValueError, match="synchronous quorum"):
+        DiLoCo(manager, model, optim.SGD(model.parameters()), optim.SGD(model.parameters()), 2)
+
+
+@pytest.mark.parametrize("outer_kind", ["sgd_nesterov", "adam"])
+def test_diloco_matches_reference_loop_with_identity_allreduce(cpu_ops, outer_kind):
+    """One replica, allreduce = identity (a mocked Manager whose allreduce returns the
+    tensor): the wrapper must leave the model exactly where the reference's loop would."""
+    torch.manual_seed(3)
+    model = SimpleModel()
+    twin = SimpleModel()
+    twin.load_state_dict(model.state_dict())
+
+    def make_outer(m):
+        if outer_kind == "adam":
+            return optim.Adam(m.parameters(), lr=1e-2)  # not fusable: optimizer.step() path
+        return optim.SGD(m.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = False
+    manager.should_commit.return_value = True
+
+    def allreduce(t):
+        f = Future()
+        f.set_result(t)
+        return f
+
+    manager.allreduce.side_effect = allreduce
+    inner, outer = optim.SGD(model.parameters(), lr=0.1), make_outer(model)
+    twin_inner, twin_outer = optim.SGD(twin.parameters(), lr=0.1), make_outer(twin)
+    twin_backup = [p.data.clone() for p in twin.parameters()]
+    pg = O.make_gloo_world1()
+    with DiLoCo(manager, model, inner, outer, sync_every=2):
+        for step in range(6):
+            x = torch.rand(2, 3)
+            for m, o in ((model, inner), (twin, twin_inner)):
+                o.zero_grad()
+                m(x).mean().backward()
+                o.step()
+            if step % 2 == 1:
+                O.diloco_reference_loop_(pg, list(twin.parameters()), twin_backup, [], twin_outer, 1)
+            for a, b in zip(model.parameters(), twin.parameters()):
+                assert_bits_equal(a.data, b.data, f"step {step}")
+    fused_calls = [c for c in cpu_ops.calls if c == "mt_outer_sgd"]
+    assert (len(fused_calls) == 3) == (outer_kind == "sgd_nesterov")
+
+
+def test_diloco_no_commit_discards_the_step(cpu_ops):
+    model = SimpleModel()
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = False
+    manager.should_commit.return_value = False
+    og = {k: v.clone() for k, v in model.state_dict().items()}
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        _train_step(model, inner)
+        torch.testing.assert_close(dict(model.state_dict()), og)
+        torch.testing.assert_close(diloco._backup_parameters, _params_dict(model))
+        assert outer.state_dict()["state"] == {}  # no momentum state from a discarded step
+        assert all(p.grad is None for p in model.parameters())
+
+
+# ---------------------------------------------------------------------------
+# Manager: torchft/manager_test.py (allreduce numerics, errors, participation)
+# ---------------------------------------------------------------------------
+
+class ScriptedQuorum(QuorumClient):
+    def __init__(self, result: QuorumResult) -> None:
+        self.result = result
+        self.votes = []
+
+    def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+        return self.result
+
+    def should_commit(self, rank, step, should_commit, timeout):
+        self.votes.append(should_commit)
+        return should_commit
+
+
+def _manager(pg=None, quorum=None, **kw) -> Manager:
+    pg = pg if pg is not None else create_autospec(ProcessGroup)
+    return Manager(pg=pg, min_replica_size=kw.pop("min_replica_size", 2),
+                   quorum_client=quorum or ScriptedQuorum(QuorumResult(
+                       quorum_id=123, replica_rank=1, replica_world_size=2, max_step=1,
+                       max_rank=1, max_world_size=2)), **kw)
+
+
+def test_manager_numerics(cpu_ops):
+    """torchft/manager_test.py:520-543."""
+    manager = _manager()
+    manager._quorum_future = MagicMock()
+    manager._participating_rank = 1
+    manager._participating_world_size = 5
+    assert manager.num_participants() == 5
+    manager._pg.allreduce.return_value = _DummyWork(None)
+    assert manager.is_participating()
+    result = manager.allreduce(torch.tensor([1.0])).value()
+    torch.testing.assert_close(result, torch.tensor([1.0 / 5]))
+    manager._healing = True
+    assert not manager.is_participating()
+    result = manager.allreduce(torch.tensor([1.0])).value()
+    torch.testing.assert_close(result, torch.tensor([0.0]))
+    manager.shutdown(wait=False)
+
+
+def test_allreduce_future_resolves_to_the_same_tensor(cpu_ops):
+    manager = _manager()
+    manager._pg.allreduce.return_value = _DummyWork(None)
+    manager.start_quorum()
+    t = torch.tensor([4.0, 8.0])
+    fut = manager.allreduce(t)
+    assert fut.wait() is t
+    torch.testing.assert_close(t, torch.tensor([2.0, 4.0]))
+    assert manager._pending_work == [fut]
+    assert manager.should_commit()
+    assert manager._pending_work == []
+    manager.shutdown(wait=False)
+
+
+def test_allreduce_error(cpu_ops):
+    """torchft/manager_test.py:338-405: errors are swallowed, latched, block the commit
+    and are cleared by the next start_quorum."""
+    manager = _manager()
+    manager._pg.allreduce.return_value = _DummyWork(None)
+    assert manager._quorum_id == -1 and manager.current_step() == 0
+    manager.start_quorum()
+    manager.allreduce(torch.tensor([1.0])).wait()
+    assert manager._pg.allreduce.call_count == 1
+    assert manager._pg.configure.call_count == 1 and manager._quorum_id == 123
+
+    manager._pg.allreduce.side_effect = RuntimeError("injected failure")
+    manager.allreduce(torch.tensor([1.0])).wait()
+    assert manager.errored()
+    manager.allreduce(torch.tensor([1.0])).wait()  # skipped
+    assert manager._pg.allreduce.call_count == 2
+    assert not manager.should_commit()
+    assert manager.errored()
+    assert manager.current_step() == 0
+
+    manager._pg.allreduce.side_effect = None
+    manager.start_quorum()
+    assert not manager.errored()
+    bad = Future()
+    bad.set_exception(RuntimeError("injected failure"))
+    work = MagicMock()
+    work.get_future.return_value = bad
+    manager._pg.allreduce.return_value = work
+    t = torch.tensor([1.0])
+    assert manager.allreduce(t).wait() is t  # completes with the input tensor
+    assert manager.errored()
+    assert not manager.should_commit()
+
+    manager._pg.allreduce.return_value = _DummyWork(None)
+    manager.start_quorum()
+    manager.allreduce(torch.tensor([1.0])).wait()
+    assert manager.should_commit()
+    assert manager.current_step() == 1 and manager.batches_committed() == 2
+    manager.shutdown(wait=False)
+
+
+@pytest.mark.parametrize("rank", [1, 2])
+def test_quorum_fixed_world_size(cpu_ops, rank):
+    """torchft/manager_test.py:407-442: spares beyond min_replica_size do not participate."""
+    q = QuorumResult(quorum_id=123, replica_rank=rank, replica_world_size=3, max_step=1,
+                     max_rank=rank, max_world_size=3)
+    manager = _manager(quorum=ScriptedQuorum(q), min_replica_size=2,
+                       world_size_mode=WorldSizeMode.FIXED_WITH_SPARES)
+    manager._pg.allreduce.return_value = _DummyWork(None)
+    manager.start_quorum()
+    t = torch.tensor([1.0])
+    manager.allreduce(t).wait()
+    assert manager.is_participating() == (rank != 2)
+    assert manager.num_participants() == 2
+    torch.testing.assert_close(t, torch.tensor([0.5 if rank != 2 else 0.0]))
+    assert manager.should_commit()
+    assert manager.batches_committed() == 2 and manager.current_step() == 1
+    manager.shutdown(wait=False)
+
+
+def test_async_quorum_counts_only_up_to_date_replicas(cpu_ops):
+    """torchft/manager.py:452-468: async quorum uses (max_rank, max_world_size); a replica
+    that is behind (max_rank None) contributes zeros; sync quorum uses the whole group."""
+    q = QuorumResult(quorum_id=1, replica_rank=1, replica_world_size=3, max_step=20,
+                     max_rank=None, max_world_size=2)
+    m = _manager(quorum=ScriptedQuorum(q), use_async_quorum=True, min_replica_size=1)
+    m._pg.allreduce.return_value = _DummyWork(None)
+    m.start_quorum(allow_heal=False)
+    m.wait_quorum()
+    assert not m.is_participating() and m.num_participants() == 2
+    t = torch.tensor([1.0])
+    m.allreduce(t).wait()
+    torch.testing.assert_close(t, torch.zeros(1))
+    m.shutdown(wait=False)
+    m = _manager(quorum=ScriptedQuorum(q), use_async_quorum=False, min_replica_size=1)
+    m.start_quorum()
+    assert m.is_participating() and m.num_participants() == 3
+    m.shutdown(wait=False)
+
+
+def test_not_enough_participants_blocks_commit(cpu_ops):
+    q = QuorumResult(quorum_id=1, replica_rank=0, replica_world_size=1, max_step=0, max_rank=0,
+                     max_world_size=1)
+    m = _manager(quorum=ScriptedQuorum(q), min_replica_size=2)
+    m.start_quorum()
+    assert not m.should_commit()
+    assert m._client.votes == [False]
+    m.shutdown(wait=False)
+
+
+def test_manager_wrap_future_and_timeout():
+    """torchft/manager_test.py:486-518."""
+    manager = _manager()
+    assert not manager.errored()
+    fut = Future()
+    wrapped = manager.wrap_future(fut, 2)
+    fut.set_exception(RuntimeError("injected failure"))
+    assert wrapped.value() == 2
+    assert manager.errored() is not None
+    assert manager._pending_work == [wrapped]
+    manager.shutdown(wait=False)
+
+    manager = _manager(timeout=timedelta(seconds=0.01))
+    wrapped = manager.wrap_future(Future(), 2)
+    wrapped.wait()
+    error = manager.errored()
+    assert isinstance(error, TimeoutError)
+    assert "future did not complete within" in str(error) and "0.01" in str(error)
+    manager.shutdown(wait=False)
+
+
+def test_manager_state_dict_round_trip():
+    m = _manager()
+    m.load_state_dict({"step": 7, "batches_committed": 21})
+    assert m.current_step() == 7 and m.batches_committed() == 21
+    assert m.state_dict() == {"step": 7, "batches_committed": 21}
+    m.set_state_dict_fns(lambda sd: None, lambda: {"w": 1})
+    assert m._manager_state_dict() == {"user": {"w": 1}, "torchft": m.state_dict()}
+    m.shutdown(wait=False)
+
+
+def test_heal_applies_the_recovered_state(cpu_ops):
+    """torchft/manager.py:492-543 with an in-process transport: a healing replica loads the
+    peer's state dict and step before the step runs (sync quorum)."""
+    server = CheckpointServer(timeout=timedelta(seconds=10))
+    server.send_checkpoint([1], 20, {"user": {"w": 5}, "torchft": {"step": 20, "batches_committed": 40}},
+                           timedelta(seconds=10))
+
+    class Healing(ScriptedQuorum):
+        def checkpoint_metadata(self, address, rank, timeout):
+            assert address == "peer manager"
+            return server.metadata()
+
+    q = QuorumResult(quorum_id=5, replica_rank=1, replica_world_size=2, max_step=20, max_rank=None,
+                     max_world_size=1, heal=True, recover_src_rank=0,
+                     recover_src_manager_address="peer manager")
+    loaded = []
+    mine = CheckpointServer(timeout=timedelta(seconds=10))
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=loaded.append, state_dict=lambda: {},
+                min_replica_size=1, use_async_quorum=False, quorum_client=Healing(q),
+                checkpoint_transport=mine)
+    m.start_quorum()
+    assert loaded == [{"w": 5}]
+    assert m.current_step() == 20 and m.batches_committed() == 40
+    assert not m._healing and m.is_participating()
+    m.shutdown()
+    server.shutdown()
+
+
+# ---------------------------------------------------------------------------
+# Local replica group
+# ---------------------------------------------------------------------------
+
+def test_local_replicas_order_and_masks(cpu_ops):
+    pg = ProcessGroupLocalReplicas(rank=1, world_size=3, peer_participating=[True, False])
+    mine = torch.tensor([10.0])
+    peers = [torch.tensor([1.0]), torch.tensor([100.0])]
+    pg.register_peers(mine, peers)
+    replicas, mask = pg.ordered(mine, True)
+    assert [float(r) for r in replicas] == [1.0, 10.0, 100.0]
+    assert mask == 0b011
+    _, mask = pg.ordered(mine, False)
+    assert mask == 0b001
+    pg.allreduce([mine], torch.distributed.ReduceOp.SUM).wait()
+    torch.testing.assert_close(mine, torch.tensor([11.0]))  # peer 2 contributes zeros
+    with pytest.raises(KeyError):
+        pg.peers_of(torch.tensor([0.0]))
+    with pytest.raises(ValueError):
+        pg.configure("addr", 0, 3)
+    pg.configure("addr", 1, 3)
+    with pytest.raises(NotImplementedError):
+        pg.allreduce([mine], torch.distributed.ReduceOp.MAX)
+    assert pg.size() == 3 and pg.getBackendName() == "torchft-local-replicas"
+
+
+def _replica_world(model: nn.Module, n: int):
+    """n-1 peer models + the lookup that pairs their parameters with the local ones."""
+    import copy
+
+    peers = [copy.deepcopy(model) for _ in range(n - 1)]
+    index = {}
+
+    def refresh():
+        index.clear()
+        for k, p in enumerate(model.parameters()):
+            for t in (p.data, p.grad):
+                if t is not None:
+                    index[t.data_ptr()] = (k, t is p.grad)
+
+    def lookup(t):
+        refresh()
+        k, is_grad = index[t.data_ptr()]
+        out = []
+        for peer in peers:
+            q = list(peer.parameters())[k]
+            out.append(q.grad if is_grad else q.data)
+        return out
+
+    return peers, lookup
+
+
+@pytest.mark.parametrize("commit", [True, False])
+def test_diloco_fused_on_local_replicas(cpu_ops, commit):
+    """This package's Manager + local replica group: the sync is ONE fused launch (or one
+    restore when the commit is refused) and matches the checker."""
+    torch.manual_seed(0)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 3)
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=3, peer_lookup=lookup)
+
+    class Vote(StaticQuorum):
+        def should_commit(self, rank, step, should_commit, timeout):
+            return should_commit and commit
+
+    manager = Manager(pg=pg, min_replica_size=1, use_async_quorum=False,
+                      quorum_client=Vote(0, 3))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    backup = [p.data.clone() for p in model.parameters()]
+    bufs = None
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        for step in range(2):
+            for k, peer in enumerate(peers):  # peers drift on their own
+                for q, b in zip(peer.parameters(), backup):
+                    q.data.copy_(b + 1e-3 * (k + 1) * torch.randn_like(b))
+            cpu_ops.calls.clear()
+            inner.zero_grad()
+            model(torch.rand(2, 3)).mean().backward()
+            before = [p.data.clone() for p in model.parameters()]
+            # what the sync must produce, from the state just before inner.step() syncs
+            grads = [p.grad.clone() for p in model.parameters()]
+            local = [b_ - 0.1 * g for b_, g in zip(before, grads)]
+            want = O.diloco_perform_sync(
+                [local] + [[q.data.clone() for q in peer.parameters()] for peer in peers],
+                backup, bufs, [True] * 3, 3, commit, lr=0.7, momentum=0.9, nesterov=True)
+            inner.step()
+            for p, w in zip(model.parameters(), want["params"]):
+                assert_bits_equal(p.data, w, f"step {step}")
+            for (name, b_), w in zip(diloco._backup_parameters.items(), want["backup"]):
+                assert_bits_equal(b_, w, f"backup {name}")
+            if commit:
+                assert cpu_ops.calls.count("mt_diloco_outer") == 1
+                assert "mt_pseudograd_avg" not in [c for c in cpu_ops.calls[:1]]
+                for p, w in zip(model.parameters(), want["momentum"]):
+                    assert_bits_equal(outer.state[p]["momentum_buffer"], w)
+                backup, bufs = want["backup"], want["momentum"]
+            else:
+                assert "mt_diloco_outer" not in cpu_ops.calls
+                assert outer.state_dict()["state"] == {}
+            assert manager.current_step() == (step + 1 if commit else 0)
+    manager.shutdown(wait=False)
+
+
+def test_local_sgd_fused_on_local_replicas(cpu_ops):
+    torch.manual_seed(1)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 2)
+    for peer in peers:
+        for q in peer.parameters():
+            q.data.add_(0.01)
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    manager = Manager(pg=pg, min_replica_size=1, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1) as local_sgd:
+        model(torch.rand(2, 3)).mean().backward()
+        local = [p.data - 0.1 * p.grad for p in model.parameters()]
+        want = O.localsgd_perform_sync(
+            [local, [q.data.clone() for q in peers[0].parameters()]],
+            [b.clone() for b in local_sgd._backup_parameters.values()], [True, True], 2, True)
+        optimizer.step()
+        for p, w in zip(model.parameters(), want["params"]):
+            assert_bits_equal(p.data, w)
+        torch.testing.assert_close(local_sgd._backup_parameters, _params_dict(model))
+        assert cpu_ops.calls.count("mt_reduce_avg") == 1  # average + backup refresh, one launch
+    manager.shutdown(wait=False)
+
+
+# ---------------------------------------------------------------------------
+# torchft/ddp_test.py, torchft/optim_test.py
+# ---------------------------------------------------------------------------
+
+def test_pure_ddp():
+    manager = create_autospec(Manager)
+    m = PureDistributedDataParallel(manager, nn.Linear(3, 4))
+    m(torch.rand(2, 3)).mean().backward()
+    for p in m.parameters():
+        assert p.grad is not None
+    assert manager.allreduce.call_count == len(list(m.parameters()))
+
+
+def test_ddp():
+    manager = create_autospec(Manager)
+    call_count = 0
+
+    def allreduce(tensor: torch.Tensor) -> Future:
+        nonlocal call_count
+        call_count += 1
+        fut = Future()
+        fut.set_result(tensor)
+        return fut
+
+    manager.allreduce = allreduce
+    m = DistributedDataParallel(manager, nn.Linear(3, 4))
+    m(torch.rand(2, 3)).mean().backward()
+    for p in m.parameters():
+        assert p.grad is not None
+    assert call_count >= 1
+
+
+def test_ddp_buckets_follow_the_reducer_rule():
+    sizes = [p * 4 for p in (2_097_152, 2_048, 4_194_304, 2_048, 20_480, 10)]
+    assert compute_bucket_assignment(sizes) == [[1, 2, 3, 4, 5], [0]]
+    assert compute_bucket_assignment(sizes) == O.bucket_assignment([s // 4 for s in sizes], 4)
+    metas = [torch.empty(s, dtype=torch.bfloat16, device="meta") for _, s in workloads.llama3_8b_shapes()]
+    got = compute_bucket_assignment([m.numel() * 2 for m in metas])
+    idx, _ = torch.distributed._compute_bucket_assignment_by_size(
+        metas, [1024 * 1024, 25 * 1024 * 1024], [False] * len(metas))
+    assert got == list(reversed(idx))
+
+
+def test_optimizer_wrapper():
+    """torchft/optim_test.py:18-50."""
+    manager = create_autospec(Manager)
+    m = nn.Linear(3, 4)
+    base = optim.AdamW(m.parameters())
+    wrapped = OptimizerWrapper(manager, base)
+    wrapped.add_param_group({"params": [nn.Parameter(torch.zeros(1))], "lr": 1})
+    assert wrapped.state_dict() == base.state_dict()
+    wrapped.zero_grad()
+    assert manager.start_quorum.call_count == 1
+    manager.should_commit.return_value = True
+    wrapped.step()
+    manager.should_commit.return_value = False
+    wrapped.step()
+    assert manager.should_commit.call_count == 2
+    assert wrapped.param_groups is base.param_groups and wrapped.state is base.state
+
+
+# ---------------------------------------------------------------------------
+# torchft/checkpointing_test.py
+# ---------------------------------------------------------------------------
+
+def test_checkpoint_server():
+    expected = {"state": "dict", "nested": {"step": 3, "lr": [0.1, (1, 2)]}}
+    server = CheckpointServer(timeout=timedelta(seconds=10))
+    server.send_checkpoint(dst_ranks=[], step=1234, state_dict=expected, timeout=timedelta(seconds=10))
+    metadata = server.metadata()
+    out = server.recv_checkpoint(src_rank=0, metadata=metadata, step=1234, timeout=timedelta(seconds=10))
+    assert out == expected
+    with pytest.raises(urllib.error.URLError, match="urlopen error"):
+        server.recv_checkpoint(src_rank=0, metadata=metadata, step=1234, timeout=timedelta(seconds=0.0))
+    server.send_checkpoint(dst_ranks=[], step=2345, state_dict=expected, timeout=timedelta(seconds=10))
+    with pytest.raises(urllib.error.HTTPError, match="Error 400"):
+        server.recv_checkpoint(src_rank=0, metadata=metadata, step=1234, timeout=timedelta(seconds=10))
+    server.shutdown()
+
+
+def test_checkpoint_server_cpu_tensors_travel_in_the_header():
+    state = {"w": torch.arange(6, dtype=torch.float32).view(2, 3), "n": 3}
+    server = CheckpointServer(timeout=timedelta(seconds=10))
+    server.send_checkpoint([], 1, state, timedelta(seconds=10))
+    out = server.recv_checkpoint(0, server.metadata(), 1, timedelta(seconds=10))
+    assert out["n"] == 3 and torch.equal(out["w"], state["w"])
+    server.shutdown()
+
+
+def test_checkpoint_server_locking():
+    server = CheckpointServer(timeout=timedelta(seconds=10))
+    assert server._checkpoint_lock.locked() and server._disallowed and server._step == -1
+    server.allow_checkpoint(1)
+    assert not server._checkpoint_lock.locked() and not server._disallowed and server._step == 1
+    server.allow_checkpoint(2)
+    assert server._step == 2
+    server.disallow_checkpoint()
+    server.disallow_checkpoint()
+    assert server._checkpoint_lock.locked() and server._disallowed
+    server.shutdown()
+
+
+def test_timed_acquire():
+    lock = threading.Lock()
+    with _timed_acquire(lock, timedelta(seconds=10)):
+        assert lock.locked()
+    assert not lock.locked()
+    lock.acquire()
+    with pytest.raises(TimeoutError, match=r"timed out acquiring lock after 0:00:00"):
+        with _timed_acquire(lock, timedelta(seconds=0.0)):
+            pass
+    assert lock.locked()
+
+
+# ---------------------------------------------------------------------------
+# No CPU path
+# ---------------------------------------------------------------------------
+
+def test_kernels_refuse_cpu_tensors():
+    from torchft_amd import ops
+
+    x = torch.zeros(8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.reduce_avg_(x, [x])
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.mt_copy([x], [x.clone()])
+    model = SimpleModel()
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = False
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    with DiLoCo(manager, model, inner, optim.SGD(model.parameters(), lr=0.7), sync_every=1):
+        model(torch.rand(2, 3)).mean().backward()
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            inner.step()

@@ -18,9 +18,10 @@ import torch  # noqa: F401  (must precede loading the library, see module docstr
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchft_amd.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 MAX_REPLICAS = 8
-MIN_CHUNK_ELEMS = 1024
+MIN_CHUNK_ELEMS = 8192
+MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
 
 TFT_F32 = 0
 TFT_BF16 = 1
@@ -31,6 +32,7 @@ class MtTable(Structure):
         ("ptrs", c_void_p),
         ("numel", c_void_p),
         ("chunk_start", c_void_p),
+        ("chunk_tensor", c_void_p),
         ("n_tensors", c_uint32),
         ("n_cols", c_uint32),
         ("chunk_elems", c_uint32),
@@ -53,7 +55,10 @@ class SgdParams(Structure):
 SIGNATURES = {
     "tft_abi_version": (c_int, []),
     "tft_last_error": (c_char_p, []),
-    "tft_mt_plan": (c_int64, [POINTER(c_uint64), c_uint32, c_uint32, POINTER(c_uint32)]),
+    "tft_mt_plan": (
+        c_int64,
+        [POINTER(c_uint64), c_uint32, c_uint32, POINTER(c_uint32), POINTER(c_uint32)],
+    ),
     "tft_default_chunk_elems": (c_uint32, [c_int]),
     "tft_reduce_avg": (
         c_int,

@@ -1,0 +1,176 @@
+"""Fault-tolerant DistributedDataParallel: gradient buckets averaged through the Manager.
+
+``DistributedDataParallel`` and ``PureDistributedDataParallel`` keep the
+reference's behaviour (torchft/ddp.py:32-97): torch's Reducer flattens the
+gradients into buckets and the communication hook hands every bucket buffer to
+``manager.allreduce``, which runs as one HIP kernel (zero / sum / divide fused)
+on a process group that offers it.
+
+``GradBucketAverager`` is the MI355X-native form of the same step for callers
+that own the gradient tensors of all replicas on one GPU (the simulated
+N-replica setting): it reproduces the Reducer's bucket layout, but instead of
+copying gradients into a flat buffer, reducing it and copying them back out, it
+addresses every bucket through its per-parameter views in one tensor table, so
+flatten and unflatten cost no memory traffic at all.
+"""
+
+# No postponed evaluation of annotations here: torch checks that the communication
+# hook annotates its bucket argument with the dist.GradBucket class itself.
+from typing import TYPE_CHECKING, Dict, List, Optional, Sequence
+
+import torch
+import torch.distributed as dist
+from torch import nn
+from torch.nn import parallel
+
+from . import ops
+from .multi_tensor import TensorTable
+from .process_group import ProcessGroupDummy
+
+if TYPE_CHECKING:
+    from .manager import Manager
+
+DEFAULT_FIRST_BUCKET_BYTES = 1024 * 1024
+DEFAULT_BUCKET_CAP_BYTES = 25 * 1024 * 1024
+
+
+class DistributedDataParallel(parallel.DistributedDataParallel):
+    """torch's DDP with its collectives replaced by ``manager.allreduce``
+    (torchft/ddp.py:32-71).  A dummy process group absorbs the constructor's
+    collectives; ``find_unused_parameters=True`` stops the Reducer from rebuilding
+    its buckets after the first step, which would make a recovering replica's bucket
+    layout differ from its peers'."""
+
+    def __init__(self, manager: "Manager", module: nn.Module, **kwargs: object) -> None:
+        pg = ProcessGroupDummy(0, 1)
+        super().__init__(
+            module,
+            process_group=pg,
+            find_unused_parameters=True,
+            **kwargs,  # type: ignore[arg-type]
+        )
+        self.register_comm_hook(manager, self._comm_hook)
+
+    @staticmethod
+    def _comm_hook(
+        state: "Manager", bucket: dist.GradBucket
+    ) -> torch.futures.Future[torch.Tensor]:
+        return state.allreduce(bucket.buffer())
+
+
+class PureDistributedDataParallel(nn.Module):
+    """DDP without a Reducer: one ``manager.allreduce`` per gradient as soon as it has
+    been accumulated (torchft/ddp.py:74-97)."""
+
+    def __init__(self, manager: "Manager", module: nn.Module) -> None:
+        super().__init__()
+        self.module = module
+
+        def post_grad_hook(p: torch.Tensor) -> None:
+            if p.grad is not None:
+                manager.allreduce(p.grad)
+
+        for p in module.parameters():
+            p.register_post_accumulate_grad_hook(post_grad_hook)
+
+    def forward(self, *args: object) -> object:
+        return self.module(*args)
+
+
+def compute_bucket_assignment(
+    sizes_bytes: Sequence[int],
+    first_cap: int = DEFAULT_FIRST_BUCKET_BYTES,
+    cap: int = DEFAULT_BUCKET_CAP_BYTES,
+) -> List[List[int]]:
+    """Bucket layout of torch's Reducer for parameters of one dtype on one device, in
+    firing order: parameters are taken in declaration order, a bucket closes once it
+    holds at least its cap (``first_cap`` for the first, ``cap`` afterwards), tensors
+    are never split, and the list is reversed because gradients arrive back to front."""
+    buckets: List[List[int]] = []
+    open_bucket: List[int] = []
+    held = 0
+    limit = first_cap
+    for i, nbytes in enumerate(sizes_bytes):
+        open_bucket.append(i)
+        held += nbytes
+        if held >= limit:
+            buckets.append(open_bucket)
+            open_bucket, held, limit = [], 0, cap
+    if open_bucket:
+        buckets.append(open_bucket)
+    buckets.reverse()
+    return buckets
+
+
+class GradBucketAverager:
+    """Averages the gradients of N replicas bucket by bucket without materialising
+    the buckets.
+
+    ``replica_grads[r][i]`` is gradient i of replica r (all on one GPU, one dtype:
+    fp32 or bf16; bf16 is accumulated in fp32).  ``out_grads[i]`` receives the
+    average; it may be one of the replicas' gradient lists (in place, as DDP does).
+    ``average_bucket(b)`` is what a communication hook does for bucket b;
+    ``average_all()`` issues every bucket in firing order.
+    """
+
+    def __init__(
+        self,
+        out_grads: Sequence[torch.Tensor],
+        replica_grads: Sequence[Sequence[torch.Tensor]],
+        first_cap: int = DEFAULT_FIRST_BUCKET_BYTES,
+        cap: int = DEFAULT_BUCKET_CAP_BYTES,
+    ) -> None:
+        if not replica_grads or any(len(g) != len(out_grads) for g in replica_grads):
+            raise ValueError("every replica needs one gradient per output gradient")
+        self.out_grads = list(out_grads)
+        self.replica_grads = [list(g) for g in replica_grads]
+        sizes = [g.numel() * g.element_size() for g in self.out_grads]
+        self.buckets = compute_bucket_assignment(sizes, first_cap, cap)
+        self._tables: List[TensorTable] = [
+            ops.reduce_avg_table(
+                [[self.out_grads[i] for i in bucket]],
+                [[g[i] for i in bucket] for g in self.replica_grads],
+            )
+            for bucket in self.buckets
+        ]
+        self._whole: Optional[TensorTable] = None
+
+    def bucket_offsets(self, b: int) -> List[int]:
+        """Element offset each gradient of bucket b would have in the flat bucket."""
+        offs, off = [], 0
+        for i in self.buckets[b]:
+            offs.append(off)
+            off += self.out_grads[i].numel()
+        return offs
+
+    def average_bucket(
+        self, b: int, participate_mask: Optional[int] = None, num_participants: Optional[int] = None
+    ) -> None:
+        bucket = self.buckets[b]
+        ops.mt_reduce_avg(
+            [[self.out_grads[i] for i in bucket]],
+            [[g[i] for i in bucket] for g in self.replica_grads],
+            participate_mask,
+            num_participants,
+            table=self._tables[b],
+        )
+
+    def average_all(
+        self, participate_mask: Optional[int] = None, num_participants: Optional[int] = None
+    ) -> None:
+        for b in range(len(self.buckets)):
+            self.average_bucket(b, participate_mask, num_participants)
+
+    def average_whole_model(
+        self, participate_mask: Optional[int] = None, num_participants: Optional[int] = None
+    ) -> None:
+        """Every bucket in ONE launch (for callers that average after backward has
+        finished instead of overlapping with it)."""
+        order = [i for bucket in self.buckets for i in bucket]
+        self._whole = ops.mt_reduce_avg(
+            [[self.out_grads[i] for i in order]],
+            [[g[i] for i in order] for g in self.replica_grads],
+            participate_mask,
+            num_participants,
+            table=self._whole,
+        )

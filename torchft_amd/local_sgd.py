@@ -1,0 +1,390 @@
+"""LocalSGD and DiLoCo with the synchronisation step fused into multi-tensor HIP launches.
+
+Same classes, constructor arguments, hooks and attributes as the reference
+(torchft/local_sgd.py:26-239): a context manager that counts optimizer steps and
+every ``sync_every`` steps starts a quorum, synchronises the replicas through the
+Manager and commits or rolls back.  What differs is how the work is issued:
+
+* the reference runs five Python loops with one or more kernels per parameter
+  tensor (subtract, all-reduce, divide, restore, SGD, save); here each of those
+  loops is one launch over a tensor table, and with this package's Manager on a
+  process group that exposes the replicas' buffers the whole DiLoCo step (all
+  loops) is a single launch;
+* the backup copy defaults to the parameters' own GPU instead of pinned host
+  memory (``backup_device=None``): the kernels need it in HBM, and 288 GB holds
+  it.  ``backup_device=torch.device("cpu")`` is still accepted by LocalSGD (plain
+  DMA copies); DiLoCo needs the backup on the device, as the reference's
+  ``p.data - backup`` does for GPU parameters.
+
+With a Manager that is not this package's (for instance a mock) the per-parameter
+``manager.allreduce`` contract is kept call for call.
+"""
+
+from __future__ import annotations
+
+import logging
+from types import TracebackType
+from typing import Dict, List, Optional, Sequence, Tuple, Type
+
+import torch
+from torch import nn, optim
+from torch.utils.hooks import RemovableHandle
+
+from . import ops
+from .manager import Manager
+from .multi_tensor import TensorTable
+
+logger: logging.Logger = logging.getLogger(__name__)
+
+
+def _is_native_manager(manager: object) -> bool:
+    # a create_autospec(Manager) double passes isinstance() but is not a subclass instance
+    return issubclass(type(manager), Manager)
+
+
+class LocalSGD:
+    """Periodic weight averaging across replicas (https://arxiv.org/pdf/1805.09767),
+    fault tolerant: if anything fails between two syncs the parameters roll back to
+    the backup taken at the last successful sync (torchft/local_sgd.py:26-175)."""
+
+    def __init__(
+        self,
+        manager: Manager,
+        model: nn.Module,
+        optimizer: optim.Optimizer,
+        sync_every: int,
+        backup_device: Optional[torch.device] = None,
+        pin_memory: bool = True,
+    ) -> None:
+        super().__init__()
+        self._manager = manager
+        self._model = model
+        self._local_optimizer = optimizer
+        self._local_step = 0
+        self._sync_every = sync_every
+        assert sync_every >= 1, "sync_every must be greater than or equal to 1"
+        self._backup_parameters: Dict[str, torch.Tensor] = {}
+        for name, p in self._model.named_parameters():
+            device = backup_device if backup_device is not None else p.device
+            t = torch.empty(*tuple(p.shape), dtype=p.dtype, device=device)
+            if pin_memory and t.device == torch.device("cpu") and torch.cuda.is_available():
+                t = t.pin_memory()
+            self._backup_parameters[name] = t
+        self._hooks: List[RemovableHandle] = []
+        self._tables: Dict[str, TensorTable] = {}
+        # the first sync needs a valid backup
+        self._save_parameters()
+
+    # -- context manager / hook ---------------------------------------------
+    def __enter__(self) -> "LocalSGD":
+        self._hooks.append(self._local_optimizer.register_step_post_hook(self._step_post_hook))
+        return self
+
+    def __exit__(
+        self,
+        exc_type: Optional[Type[BaseException]],
+        exc_value: Optional[BaseException],
+        traceback: Optional[TracebackType],
+    ) -> bool:
+        if exc_type is not None:
+            # discard the local steps since the last sync
+            self._restore_parameters()
+        for hook in self._hooks:
+            hook.remove()
+        self._hooks.clear()
+        return False  # exceptions propagate
+
+    def _step_post_hook(
+        self, _optim: optim.Optimizer, _args: List[object], _kwargs: Dict[str, object]
+    ) -> None:
+        self._local_step += 1
+        if self._local_step >= self._sync_every:
+            self.sync()
+
+    # -- tensors -------------------------------------------------------------
+    def _named(self) -> Tuple[List[str], List[torch.Tensor], List[torch.Tensor]]:
+        names, params, backups = [], [], []
+        for name, p in self._model.named_parameters():
+            assert name in self._backup_parameters
+            names.append(name)
+            params.append(p.data)
+            backups.append(self._backup_parameters[name])
+        return names, params, backups
+
+    @staticmethod
+    def _on_device(params: Sequence[torch.Tensor], backups: Sequence[torch.Tensor]) -> bool:
+        return bool(params) and all(
+            p.is_cuda and b.device == p.device and p.device == params[0].device
+            for p, b in zip(params, backups)
+        )
+
+    def _copy(self, key: str, dsts: List[torch.Tensor], srcs: List[torch.Tensor], blocking: bool) -> None:
+        if self._on_device(dsts, srcs):
+            cached = self._tables.get(key)
+            self._tables[key] = ops.mt_copy(dsts, srcs, table=cached)
+            return
+        for d, s in zip(dsts, srcs):  # host-resident backup: plain DMA, no arithmetic
+            d.copy_(s, non_blocking=not blocking)
+
+    def _save_parameters(self) -> None:
+        """backup <- parameters (torchft/local_sgd.py:121-125), one launch."""
+        with torch.no_grad():
+            _, params, backups = self._named()
+            self._copy("save", backups, params, blocking=False)
+
+    def _restore_parameters(self) -> None:
+        """parameters <- backup (torchft/local_sgd.py:127-131), one launch."""
+        with torch.no_grad():
+            _, params, backups = self._named()
+            self._copy("restore", params, backups, blocking=True)
+
+    # -- sync ------------------------------------------------------------------
+    def sync(self) -> None:
+        """Averages the model weights across the replicas of the current quorum."""
+        self._manager.start_quorum()
+        self._perform_sync()
+        self._local_step = 0
+
+    def _fused(self, params: Sequence[torch.Tensor], backups: Sequence[torch.Tensor]) -> bool:
+        return (
+            _is_native_manager(self._manager)
+            and self._manager.supports_fused_sync()
+            and self._on_device(params, backups)
+        )
+
+    def _perform_sync(self) -> None:
+        """Average, then keep the result (commit) or roll back (torchft/local_sgd.py:151-162)."""
+        _, params, backups = self._named()
+        if self._fused(params, backups):
+            if self._manager.reduction_fails_only_at_launch():
+                # a local reduction cannot fail once launched: decide first, then average
+                # and refresh the backup in the same launch
+                if self._manager.should_commit():
+                    self._manager.allreduce_tensors(params, also_write=backups).wait()
+                    if self._manager.errored() is not None:
+                        self._restore_parameters()
+                else:
+                    self._restore_parameters()
+                return
+            self._manager.allreduce_tensors(params).wait()
+        else:
+            self._average()
+        if self._manager.should_commit():
+            self._save_parameters()
+        else:
+            self._restore_parameters()
+
+    def _average(self) -> None:
+        works = []
+        for p in self._model.parameters():
+            works.append(self._manager.allreduce(p.data.detach()))
+        for work in works:
+            work.wait()
+
+
+def _fusable_sgd(
+    optimizer: optim.Optimizer, params: Sequence[torch.Tensor]
+) -> Optional[List[Tuple[List[int], ops.OuterSGD, bool]]]:
+    """If ``optimizer`` is a plain ``torch.optim.SGD`` over exactly ``params``, returns per
+    parameter group (indices into ``params``, hyper-parameters, first_step); else None."""
+    if type(optimizer) is not optim.SGD:
+        return None
+    index = {p.data_ptr(): i for i, p in enumerate(params)}
+    plan = []
+    covered = 0
+    for group in optimizer.param_groups:
+        if group.get("maximize") or group.get("differentiable"):
+            return None
+        lr = group["lr"]
+        if isinstance(lr, torch.Tensor):
+            return None
+        idx = []
+        have_buf = []
+        for p in group["params"]:
+            i = index.get(p.data_ptr())
+            if i is None or p.dtype != torch.float32:
+                return None
+            idx.append(i)
+            have_buf.append(optimizer.state.get(p, {}).get("momentum_buffer") is not None)
+        if not idx:
+            continue
+        if any(have_buf) != all(have_buf):
+            return None
+        covered += len(idx)
+        sgd = ops.OuterSGD(
+            lr=float(lr),
+            momentum=float(group["momentum"]),
+            dampening=float(group["dampening"]),
+            weight_decay=float(group["weight_decay"]),
+            nesterov=bool(group["nesterov"]),
+        )
+        plan.append((idx, sgd, not all(have_buf)))
+    if covered != len(params):
+        return None
+    return plan
+
+
+class DiLoCo(LocalSGD):
+    """DiLoCo (https://arxiv.org/pdf/2311.08105): the replicas average their
+    pseudo-gradients ``params - backup`` and an outer optimizer applies the average
+    to the parameters restored from the backup (torchft/local_sgd.py:177-239)."""
+
+    def __init__(
+        self,
+        manager: Manager,
+        model: nn.Module,
+        inner_optimizer: optim.Optimizer,
+        outer_optimizer: optim.Optimizer,
+        sync_every: int,
+        backup_device: Optional[torch.device] = None,
+        pin_memory: bool = True,
+    ) -> None:
+        if manager._use_async_quorum:
+            raise ValueError(
+                "Using DiLoCo require synchronous quorum to be enabled. "
+                "Ensure that the manager is initialized with use_async_quorum=False"
+            )
+        super().__init__(manager, model, inner_optimizer, sync_every, backup_device, pin_memory)
+        self._outer_optimizer = outer_optimizer
+        self._grads: Optional[List[torch.Tensor]] = None
+
+    def _grad_buffers(self, params: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+        """Pseudo-gradient storage, kept across syncs (the reference allocates it anew
+        with every ``p.data - backup``)."""
+        if self._grads is None or len(self._grads) != len(params) or any(
+            g.shape != p.shape or g.device != p.device or g.dtype != p.dtype
+            for g, p in zip(self._grads, params)
+        ):
+            self._grads = [torch.empty_like(p) for p in params]
+        return self._grads
+
+    def _momentum_buffers(self, idx: Sequence[int], first: bool) -> List[torch.Tensor]:
+        """The outer SGD's momentum buffers; on the first step fresh tensors that are
+        not yet part of the optimizer state (see ``_attach_momentum``)."""
+        live = [p for p in self._model.parameters()]
+        if first:
+            return [torch.empty_like(live[i].data) for i in idx]
+        return [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
+
+    def _attach_momentum(self, idx: Sequence[int], bufs: Sequence[torch.Tensor]) -> None:
+        """After a committed first step the buffers become optimizer state, exactly where
+        torch.optim.SGD keeps them."""
+        live = [p for p in self._model.parameters()]
+        for i, buf in zip(idx, bufs):
+            self._outer_optimizer.state[live[i]]["momentum_buffer"] = buf
+
+    def _outer_step(
+        self,
+        params: List[torch.Tensor],
+        backups: List[torch.Tensor],
+        grads: List[torch.Tensor],
+        plan: Optional[List[Tuple[List[int], ops.OuterSGD, bool]]],
+    ) -> None:
+        """Committed: apply the outer optimizer to the restored parameters and refresh the
+        backup (torchft/local_sgd.py:221-224)."""
+        if plan is None:
+            self._outer_optimizer.step()
+            self._save_parameters()
+            return
+        for gi, (idx, sgd, first) in enumerate(plan):
+            bufs = self._momentum_buffers(idx, first) if sgd.momentum != 0.0 else None
+            key = f"outer_sgd/{gi}"
+            self._tables[key] = ops.mt_outer_sgd(
+                [params[i] for i in idx],
+                [backups[i] for i in idx],
+                bufs,
+                [grads[i] for i in idx],
+                sgd,
+                first,
+                table=self._tables.get(key),
+            )
+            if first and bufs is not None:
+                self._attach_momentum(idx, bufs)
+
+    def _perform_sync(self) -> None:
+        """Pseudo-gradients, their average over the replicas, restore, and (on commit)
+        the outer step plus backup refresh (torchft/local_sgd.py:205-225)."""
+        _, params, backups = self._named()
+        if not self._on_device(params, backups):
+            raise RuntimeError(
+                "DiLoCo needs parameters and backup on one GPU (the kernels have no CPU path); "
+                "construct it with backup_device=None or the parameters' device"
+            )
+        live = list(self._model.parameters())
+        plan = _fusable_sgd(self._outer_optimizer, params)
+        fused = self._fused(params, backups)
+
+        if fused and plan is not None and self._manager.reduction_fails_only_at_launch():
+            self._sync_single_launch(params, backups, plan)
+            self._outer_optimizer.zero_grad()
+            return
+
+        grads = self._grad_buffers(params)
+        if fused:
+            # pseudo-gradient, replica sum, divide and restore: one launch
+            for p, g in zip(live, grads):
+                p.grad = g
+            self._manager.pseudograd_allreduce(grads, params, backups, restore_params=True).wait()
+            if self._manager.errored() is not None:
+                self._restore_parameters()  # the launch that restores did not happen
+        else:
+            # pseudo-gradients in one launch, then the Manager contract per parameter
+            self._tables["pseudograd"] = ops.mt_pseudograd_avg(
+                grads, params, backups, [params], restore_params=False,
+                table=self._tables.get("pseudograd"),
+            )
+            for p, g in zip(live, grads):
+                p.grad = g
+            self._average_grads()
+            self._restore_parameters()
+
+        if self._manager.should_commit():
+            self._outer_step(params, backups, grads, plan)
+        self._outer_optimizer.zero_grad()
+
+    def _sync_single_launch(
+        self,
+        params: List[torch.Tensor],
+        backups: List[torch.Tensor],
+        plan: List[Tuple[List[int], ops.OuterSGD, bool]],
+    ) -> None:
+        """The reduction is local and cannot fail once launched, so the commit decision
+        can be taken first and the whole sync becomes one launch per parameter group:
+        either the fully fused step, or (no commit) a plain restore."""
+        manager = self._manager
+        manager.wait_quorum()
+        launches = []
+        if manager.errored() is None:
+            try:
+                replicas, mask = manager.replica_columns(params)
+                for gi, (idx, sgd, first) in enumerate(plan):
+                    bufs = self._momentum_buffers(idx, first) if sgd.momentum != 0.0 else None
+                    cols = dict(
+                        params=[params[i] for i in idx],
+                        backups=[backups[i] for i in idx],
+                        bufs=bufs,
+                        replicas=[[rep[i] for i in idx] for rep in replicas],
+                    )
+                    launches.append((f"fused/{gi}", idx, cols, sgd, first, mask))
+            except Exception as e:  # same latch as Manager.allreduce
+                logger.exception("got exception preparing the fused sync -- skipping: %s", e)
+                manager.report_error(e)
+        if manager.should_commit():
+            for key, idx, cols, sgd, first, mask in launches:
+                self._tables[key] = ops.mt_diloco_outer(
+                    cols["params"], cols["backups"], cols["bufs"], cols["replicas"], sgd, first,
+                    mask, manager.num_participants(), table=self._tables.get(key),
+                )
+                if first and cols["bufs"] is not None:
+                    self._attach_momentum(idx, cols["bufs"])
+        else:
+            self._restore_parameters()
+
+    def _average_grads(self) -> None:
+        """One ``manager.allreduce`` per pseudo-gradient (torchft/local_sgd.py:227-239)."""
+        works = []
+        for p in self._model.parameters():
+            assert p.grad is not None
+            works.append(self._manager.allreduce(p.grad))
+        for work in works:
+            work.wait()

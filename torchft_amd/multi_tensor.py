@@ -41,19 +41,37 @@ def require_device_tensor(t: torch.Tensor, what: str) -> None:
         raise ValueError(f"{what}: tensor of shape {tuple(t.shape)} is not contiguous")
 
 
-def plan_chunks(numel: Sequence[int], chunk_elems: int) -> np.ndarray:
-    """chunk_start[0..T] for the given sizes (host-only; computed by the C library)."""
+def plan_chunks(numel: Sequence[int], chunk_elems: int) -> Tuple[np.ndarray, np.ndarray]:
+    """(chunk_start[0..T], chunk_tensor[0..K)) for the given sizes.
+
+    Host-only; both arrays are computed by the C library (tft_mt_plan)."""
     n = len(numel)
     arr = np.asarray(numel, dtype=np.uint64)
-    out = np.zeros(n + 1, dtype=np.uint32)
-    total = _native.lib().tft_mt_plan(
-        arr.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)),
-        n,
-        chunk_elems,
-        out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)),
+    start = np.zeros(n + 1, dtype=np.uint32)
+    u64p, u32p = ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint32)
+    plan = _native.lib().tft_mt_plan
+    total = plan(arr.ctypes.data_as(u64p), n, chunk_elems, start.ctypes.data_as(u32p), None)
+    _native.check(int(total), "tft_mt_plan")
+    owner = np.zeros(max(int(total), 1), dtype=np.uint32)
+    total = plan(
+        arr.ctypes.data_as(u64p), n, chunk_elems, start.ctypes.data_as(u32p),
+        owner.ctypes.data_as(u32p),
     )
     _native.check(int(total), "tft_mt_plan")
-    return out
+    return start, owner[: int(total)]
+
+
+def pick_chunk_elems(sizes: Sequence[int], default: int, minimum: int) -> int:
+    """Largest power-of-two chunk <= default whose last-chunk padding wastes < 3% of the
+    workgroups (models made of many small tensors want small chunks)."""
+    total = sum(sizes)
+    chunk = default
+    while chunk > minimum:
+        launched = sum(-(-s // chunk) for s in sizes) * chunk
+        if launched - total <= 0.03 * total:
+            break
+        chunk //= 2
+    return chunk
 
 
 class TensorTable:
@@ -119,10 +137,17 @@ class TensorTable:
             assert self.dtype is not None
             code = dtype_code(self.dtype)
         self.dtype_code = code
-        self.chunk_elems = int(chunk_elems or _native.lib().tft_default_chunk_elems(code))
         sizes = [
             columns[0][t].numel() * (columns[0][t].element_size() if as_bytes else 1) for t in rows
         ]
+        self.chunk_elems = int(
+            chunk_elems
+            or pick_chunk_elems(
+                sizes,
+                _native.lib().tft_default_chunk_elems(code),
+                _native.MIN_CHUNK_BYTES if as_bytes else _native.MIN_CHUNK_ELEMS,
+            )
+        )
         self.numel_total = int(sum(sizes))
         # keep the tensors alive and remember their identity for cache checks
         self._keepalive = [[columns[c][t] for t in rows] for c in range(n_cols)]
@@ -130,9 +155,9 @@ class TensorTable:
         if self.n_tensors == 0:
             self.total_chunks = 0
             self._blob = None
-            self.struct = _native.MtTable(None, None, None, 0, n_cols, self.chunk_elems, 0)
+            self.struct = _native.MtTable(None, None, None, None, 0, n_cols, self.chunk_elems, 0)
             return
-        chunk_start = plan_chunks(sizes, self.chunk_elems)
+        chunk_start, chunk_tensor = plan_chunks(sizes, self.chunk_elems)
         self.total_chunks = int(chunk_start[-1])
         ptrs = np.empty((n_cols, self.n_tensors), dtype=np.uint64)
         for c in range(n_cols):
@@ -142,13 +167,17 @@ class TensorTable:
         ptr_bytes = ptrs.tobytes()
         numel_bytes = numel.tobytes()
         start_bytes = chunk_start.tobytes()
-        blob = np.frombuffer(ptr_bytes + numel_bytes + start_bytes, dtype=np.uint8).copy()
+        owner_bytes = chunk_tensor.tobytes()
+        blob = np.frombuffer(
+            ptr_bytes + numel_bytes + start_bytes + owner_bytes, dtype=np.uint8
+        ).copy()
         self._blob = torch.from_numpy(blob).to(self.device)
         base = self._blob.data_ptr()
         self.struct = _native.MtTable(
             base,
             base + len(ptr_bytes),
             base + len(ptr_bytes) + len(numel_bytes),
+            base + len(ptr_bytes) + len(numel_bytes) + len(start_bytes),
             self.n_tensors,
             n_cols,
             self.chunk_elems,
