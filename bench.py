@@ -1,15 +1,22 @@
 #!/usr/bin/env python3
-"""Replica-sync benchmark: the fused DiLoCo outer step on Llama-3-8B-shaped fp32 parameters.
+"""Replica-sync benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3_8b|gpt2_small]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-One step = one pass of the fused multi-tensor outer step (pseudo-gradient of N
-replicas against the backup, average, Nesterov outer SGD, backup refresh) over
-every parameter tensor, steady state (momentum buffers exist).  All inputs are
-resident in HBM before the timed region.  Prints one JSON line with params/s,
-the kernel's achieved HBM bandwidth against the 8 TB/s peak, and the
+The default workload (the headline one) is the fused DiLoCo outer step on
+Llama-3-8B-shaped fp32 parameters: one step = one pass of the fused multi-tensor
+kernel (pseudo-gradient of N replicas against the backup, average, Nesterov outer
+SGD, backup refresh) over all 291 parameter tensors, steady state (momentum
+buffers exist), everything resident in HBM before the timed region.  One JSON line
+is printed with params/s, the kernel's achieved HBM bandwidth against the 8 TB/s
+peak (HIP events around every launch, on the stream the kernel runs on), and the
 reference's CPU loop (torch CPU ops + ProcessGroupGloo, world size 1) timed on a
 bounded slice of the same workload on this box's host cores.
+
+Other workloads measure the remaining kernels of the path with the same line
+format: ``diloco_gpt2_small``, ``ddp_buckets_llama3_8b`` (bf16 gradient buckets, 4
+contributions of which 3 participate), ``checkpoint_llama3_8b`` (pack / unpack of an
+80 GB training state, plus the PCIe legs), ``localsgd_llama3_8b``.
 """
 
 from __future__ import annotations
@@ -19,6 +26,7 @@ import json
 import os
 import sys
 import time
+from typing import Callable, Dict, List, Tuple
 
 import torch
 
@@ -27,8 +35,10 @@ if REPO_ROOT not in sys.path:
     sys.path.insert(0, REPO_ROOT)
 
 HBM_PEAK_GBS = 8000.0
-N_REPLICAS = {"llama3_8b": 2, "gpt2_small": 4}
 LR, MOMENTUM = 0.7, 0.9
+HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo"
+WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
+             "checkpoint_llama3_8b", "localsgd_llama3_8b"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -36,29 +46,77 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=sorted(N_REPLICAS), default="llama3_8b")
+    ap.add_argument("--workload", choices=WORKLOADS, default=WORKLOADS[0])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=2,
                     help="decoder layers in the CPU baseline's slice of the Llama workload")
     ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="run one plain multi-tensor copy of known size before the timed loop "
+                         "(reference point for hardware-counter runs)")
+    ap.add_argument("--variant", type=int, default=0, help="launch variant (tuning; 0 = default)")
     return ap.parse_args()
 
 
-def cpu_baseline(args: argparse.Namespace) -> dict:
-    """The reference's own loop (per-tensor torch CPU ops, Gloo world size 1), timed."""
+class Timed:
+    """K steps, wall clock bracketed by synchronize, HIP events around every launch group."""
+
+    def __init__(self, steps: int, warmup: int) -> None:
+        self.steps, self.warmup = steps, warmup
+
+    def run(self, step: Callable[[], None]) -> Tuple[float, float]:
+        for _ in range(self.warmup):
+            step()
+        torch.cuda.synchronize()
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(self.steps)]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in range(self.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(self.steps):
+            starts[i].record()
+            step()
+            stops[i].record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / self.steps
+        kernel_ms = sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / self.steps
+        return wall_ms, kernel_ms
+
+
+def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1) -> Dict[str, object]:
+    achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    return {
+        "bound": "hbm",
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS,
+        "traffic": None,
+        "kernel": kernel,
+        "kernel_ms_per_step": kernel_ms,
+        "launches_per_step": launches,
+        "algorithmic_bytes_per_step": algo_bytes,
+    }
+
+
+def base_line(args, metric: str, value: float, unit: str, ms_per_step: float, dtype: str,
+              config: Dict[str, object]) -> Dict[str, object]:
+    return {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": config,
+    }
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline: the reference's loop, timed
+# ---------------------------------------------------------------------------
+
+def cpu_baseline_diloco(args, shapes, n_rep: int, sample: str) -> Dict[str, object]:
     from oracle import replica_sync as O
     from torchft_amd import workloads
 
-    if args.workload == "llama3_8b":
-        shapes = workloads.llama3_8b_shapes(args.cpu_layers, with_embeddings=False)
-        sample = (f"{args.cpu_layers} of 32 decoder layers of the Llama-3-8B workload "
-                  f"(no embeddings), {args.cpu_steps} steps after 1 warm-up")
-    else:
-        shapes = workloads.gpt2_small_shapes()
-        sample = f"full GPT-2-small workload, {args.cpu_steps} steps after 1 warm-up"
-    n_rep = N_REPLICAS[args.workload]
-    cpu = torch.device("cpu")
-    wl = workloads.make_diloco_workload(shapes, n_rep, cpu)
+    wl = workloads.make_diloco_workload(shapes, n_rep, torch.device("cpu"))
     params = [torch.nn.Parameter(t) for t in wl.replicas[0]]
     opt = torch.optim.SGD(params, lr=LR, momentum=MOMENTUM, nesterov=True)
     pg = O.make_gloo_world1()
@@ -69,13 +127,173 @@ def cpu_baseline(args: argparse.Namespace) -> dict:
         O.diloco_reference_loop_(pg, params, wl.backup, peers, opt, n_rep)
     dt = (time.perf_counter() - t0) / args.cpu_steps
     return {
-        "value": wl.n_params / dt,
-        "unit": "params/s",
-        "cores": torch.get_num_threads(),
+        "value": wl.n_params / dt, "unit": "params/s", "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": sample + f"; {wl.n_params} params, {dt * 1e3:.1f} ms/step; "
-                           f"os.cpu_count()={os.cpu_count()}",
+        "sample": f"{sample}, {args.cpu_steps} steps after 1 warm-up; {wl.n_params} params, "
+                  f"{dt * 1e3:.1f} ms/step; torch CPU ops + ProcessGroupGloo world size 1, "
+                  f"os.cpu_count()={os.cpu_count()}",
     }
+
+
+# ---------------------------------------------------------------------------
+# Workloads
+# ---------------------------------------------------------------------------
+
+def bench_diloco(args, which: str) -> Dict[str, object]:
+    from torchft_amd import ops, workloads
+    from torchft_amd.multi_tensor import TensorTable
+
+    dev = torch.device("cuda", 0)
+    if which == "llama3_8b":
+        shapes, n_rep = workloads.llama3_8b_shapes(), 2
+    else:
+        shapes, n_rep = workloads.gpt2_small_shapes(), 4
+    wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+    params = [torch.empty_like(t) for t in wl.backup]
+    bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
+    sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
+    table = TensorTable([params, wl.backup, bufs, *wl.replicas], what="bench")
+    torch.cuda.synchronize()
+    if args.calibration_copy:
+        ops.mt_copy(params, wl.backup)
+        torch.cuda.synchronize()
+
+    def step() -> None:
+        ops.mt_diloco_outer(params, wl.backup, bufs, wl.replicas, sgd, False, table=table)
+
+    wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
+    probe = len(params) // 2
+    if not torch.isfinite(params[probe]).all() or not torch.equal(params[probe], wl.backup[probe]):
+        raise RuntimeError("output check failed: parameters are not finite or differ from the backup")
+
+    n_params = wl.n_params
+    # read N replicas, backup, momentum; write momentum, parameters, backup
+    algo_bytes = n_params * (4 * n_rep + 20)
+    out = base_line(
+        args, HEADLINE_METRIC if which == "llama3_8b" else "outer-sync params/sec, GPT-2-small DiLoCo",
+        n_params / (wall_ms * 1e-3), "params/s", wall_ms, "f32",
+        {"workload": f"DiLoCo outer step, fp32, {which}-shaped params ({len(shapes)} tensors, "
+                     f"{n_params} params), {n_rep} simulated replicas, Nesterov SGD lr={LR} "
+                     f"momentum={MOMENTUM}, one fused multi-tensor launch per step",
+         "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
+    out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>")
+    if not args.no_cpu_baseline:
+        if which == "llama3_8b":
+            cpu_shapes = workloads.llama3_8b_shapes(args.cpu_layers, with_embeddings=False)
+            sample = f"{args.cpu_layers} of 32 decoder layers of the Llama-3-8B workload (no embeddings)"
+        else:
+            cpu_shapes, sample = shapes, "full GPT-2-small workload"
+        out["cpu_baseline"] = cpu_baseline_diloco(args, cpu_shapes, n_rep, sample)
+    return out
+
+
+def bench_localsgd(args) -> Dict[str, object]:
+    from torchft_amd import ops, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes, n_rep = workloads.llama3_8b_shapes(), 2
+    wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+    table = ops.reduce_avg_table([wl.replicas[0], wl.backup], wl.replicas)
+
+    def step() -> None:
+        ops.mt_reduce_avg([wl.replicas[0], wl.backup], wl.replicas, table=table)
+
+    wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
+    n_params = wl.n_params
+    out = base_line(args, "LocalSGD sync params/sec, Llama-3-8B", n_params / (wall_ms * 1e-3),
+                    "params/s", wall_ms, "f32",
+                    {"workload": "LocalSGD weight average + backup refresh, fp32, Llama-3-8B-shaped "
+                                 "params, 2 simulated replicas, one launch per step",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
+    out["roofline"] = roofline(n_params * 4 * (n_rep + 2), kernel_ms,
+                               "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>")
+    return out
+
+
+def bench_ddp_buckets(args) -> Dict[str, object]:
+    from torchft_amd import GradBucketAverager, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+    grads = workloads.make_grad_replicas(shapes, 4, dev, torch.bfloat16)
+    averager = GradBucketAverager(grads[0], grads)  # in place on replica 0, like a DDP bucket
+    mask, n = 0b0111, 3  # replica 3 is a spare: zeroed, never read
+
+    def step() -> None:
+        averager.average_all(mask, n)
+
+    wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
+    n_elems = sum(g.numel() for g in grads[0])
+    out = base_line(args, "DDP gradient-bucket average elements/sec, Llama-3-8B bf16",
+                    n_elems / (wall_ms * 1e-3), "elements/s", wall_ms, "bf16 storage, f32 accumulate",
+                    {"workload": f"bf16 gradients of Llama-3-8B ({len(shapes)} tensors, {n_elems} "
+                                 f"elements) in {len(averager.buckets)} buckets by torch's 1 MiB / 25 MiB "
+                                 "rule, 4 contributions with 3 participating, one launch per bucket "
+                                 "over per-parameter views (no flatten / unflatten passes)",
+                     "n_buckets": len(averager.buckets), "n_elements": n_elems})
+    out["roofline"] = roofline(n_elems * 2 * (3 + 1), kernel_ms,
+                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets))
+    return out
+
+
+def bench_checkpoint(args) -> Dict[str, object]:
+    from torchft_amd import state_pack, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+    state = workloads.make_training_state(shapes, dev)
+    plan = state_pack.plan_pack(state)
+    staging = torch.empty(plan.total_bytes, dtype=torch.uint8, device=dev)
+    cache: Dict[str, object] = {}
+    torch.cuda.synchronize()
+
+    def pack_step() -> None:
+        state_pack.pack(state, staging=staging, table_cache=cache)
+
+    wall_ms, pack_ms = Timed(args.steps, args.warmup).run(pack_step)
+    entries, total = list(plan.entries), plan.total_bytes
+    payload = sum(e.nbytes for e in entries)
+    # unpack into the tensors of a second state of the same layout (scatter kernel);
+    # the source state is released first: 80 GB staging + 80 GB destination stay resident
+    del state, plan
+    cache.clear()
+    torch.cuda.empty_cache()
+    from torchft_amd import ops
+
+    outs = [torch.empty(e.shape, dtype=state_pack._DTYPES[e.dtype], device=dev) for e in entries]
+    srcs = [staging[e.offset:e.offset + e.nbytes] for e in entries]
+    table = ops.mt_copy(outs, srcs)
+    _, unpack_ms = Timed(args.steps, args.warmup).run(lambda: ops.mt_copy(outs, srcs, table=table))
+    # PCIe legs through two pinned bounce buffers (bounded host memory)
+    chunk = 1 << 30
+    bounce = [torch.empty(chunk, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i, lo in enumerate(range(0, total, chunk)):
+        n = min(chunk, total - lo)
+        bounce[i % 2][:n].copy_(staging[lo:lo + n], non_blocking=True)
+    torch.cuda.synchronize()
+    d2h_s = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for i, lo in enumerate(range(0, total, chunk)):
+        n = min(chunk, total - lo)
+        staging[lo:lo + n].copy_(bounce[i % 2][:n], non_blocking=True)
+    torch.cuda.synchronize()
+    h2d_s = time.perf_counter() - t0
+    out = base_line(args, "checkpoint pack GB/s, Llama-3-8B training state",
+                    payload / (wall_ms * 1e-3) / 1e9, "GB/s (payload bytes packed per second)", wall_ms,
+                    "u8",
+                    {"workload": f"training state of Llama-3-8B: bf16 params + fp32 AdamW exp_avg / "
+                                 f"exp_avg_sq + int64 steps, {len(entries)} device tensors, "
+                                 f"{payload} bytes, one gather launch into a contiguous staging buffer",
+                     "n_tensors": len(entries), "payload_bytes": payload})
+    out["roofline"] = roofline(2 * payload, pack_ms, "mt_copy_kernel (pack)")
+    out["unpack"] = roofline(2 * payload, unpack_ms, "mt_copy_kernel (unpack)")
+    out["pcie"] = {"d2h_GBs": total / d2h_s / 1e9, "h2d_GBs": total / h2d_s / 1e9,
+                   "d2h_s": d2h_s, "h2d_s": h2d_s, "bytes": total,
+                   "note": "staging buffer through two 1 GiB pinned bounce buffers; PCIe-bound, "
+                           "reported separately from the HBM-bound kernels"}
+    return out
 
 
 def main() -> int:
@@ -88,86 +306,20 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
+    torch.cuda.set_device(0)
+    from torchft_amd import ops
 
-    from torchft_amd import ops, workloads
-    from torchft_amd.multi_tensor import TensorTable
-
-    dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
-    shapes = workloads.llama3_8b_shapes() if args.workload == "llama3_8b" else workloads.gpt2_small_shapes()
-    n_rep = N_REPLICAS[args.workload]
-    wl = workloads.make_diloco_workload(shapes, n_rep, dev)
-    params = [torch.empty_like(t) for t in wl.backup]
-    bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
-    sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
-    table = TensorTable([params, wl.backup, bufs, *wl.replicas], what="bench")
-    torch.cuda.synchronize()
-
-    def step() -> None:
-        ops.mt_diloco_outer(params, wl.backup, bufs, wl.replicas, sgd, False, table=table)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # per-launch HIP events on the stream the kernel is enqueued on (torch's current stream)
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        starts[i].record()
-        step()
-        stops[i].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
-
-    # the result must still be finite and the backup must equal the parameters
-    probe = params[len(params) // 2]
-    if not torch.isfinite(probe).all() or not torch.equal(probe, wl.backup[len(params) // 2]):
-        print("bench.py: output check failed", file=sys.stderr)
-        return 1
-
-    n_params = wl.n_params
-    bytes_per_param = 4 * n_rep + 20  # read N replicas, backup, momentum; write momentum, params, backup
-    algo_bytes = n_params * bytes_per_param
-    achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
-    out = {
-        "metric": "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo",
-        "value": n_params / (ms_per_step * 1e-3),
-        "unit": "params/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {
-            "workload": f"DiLoCo outer step, fp32, {args.workload}-shaped params "
-                        f"({len(shapes)} tensors, {n_params} params), {n_rep} simulated replicas, "
-                        f"Nesterov SGD lr={LR} momentum={MOMENTUM}, one fused multi-tensor launch per step",
-            "n_tensors": len(shapes),
-            "n_params": n_params,
-            "n_replicas": n_rep,
-        },
-        "roofline": {
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
-            "kernel": "mt_stream_kernel<F32, DilocoFusedOp<%d>>" % n_rep,
-            "kernel_ms": kernel_ms,
-            "algorithmic_bytes_per_launch": algo_bytes,
-        },
-    }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args)
+    ops.set_launch_variant(args.variant)
+    if args.workload == "diloco_llama3_8b":
+        out = bench_diloco(args, "llama3_8b")
+    elif args.workload == "diloco_gpt2_small":
+        out = bench_diloco(args, "gpt2_small")
+    elif args.workload == "ddp_buckets_llama3_8b":
+        out = bench_ddp_buckets(args)
+    elif args.workload == "checkpoint_llama3_8b":
+        out = bench_checkpoint(args)
+    else:
+        out = bench_localsgd(args)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -106,8 +106,16 @@ __device__ inline void store16(void* p, const u32x4& v) {
 }
 
 // ---------------------------------------------------------------------------
-// Locators: map a chunk index to (column base pointers, element count).
+// Locators: map a slab index to (column base pointers, element count).
 // ---------------------------------------------------------------------------
+
+// A launch of more than 2^31 work-items in one grid dimension is silently cut
+// short by the runtime, so large slab counts are laid out as a 2-D grid with a
+// bounded x extent (see grid_for); the dispatcher still hands workgroups out
+// x-fastest, i.e. in slab order.
+constexpr uint32_t kMaxGridX = 1u << 22;
+
+__device__ inline uint32_t slab_index() { return blockIdx.y * gridDim.x + blockIdx.x; }
 struct TableArgs {
   void* const* ptrs;
   const uint64_t* numel;
@@ -116,6 +124,7 @@ struct TableArgs {
   uint32_t n_tensors;
   uint32_t chunk_elems;
   uint32_t slab_shift;  // log2(slabs per chunk)
+  uint32_t total_chunks;
 };
 
 struct FlatArgs {  // one tensor, pointers carried in the kernel arguments
@@ -130,6 +139,7 @@ struct TableLocator {
   __device__ static inline uint32_t locate(const TableArgs& a, uint32_t slab, uint32_t slab_elems,
                                            uint32_t cols, char* (&ptr)[NCOL], size_t esize) {
     const uint32_t chunk = slab >> a.slab_shift;
+    if (chunk >= a.total_chunks) return 0;  // padding of the 2-D grid
     const uint32_t sub = slab & ((1u << a.slab_shift) - 1u);
     const uint32_t t = a.chunk_tensor[chunk];
     const uint64_t numel = a.numel[t];
@@ -244,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_
   const uint32_t wmask = op.wmask();
   char* ptr[NCOL];
   const uint32_t n =
-      Loc::locate(args, blockIdx.x, kSlab, rmask | wmask, ptr, sizeof(typename E::elem_t));
+      Loc::locate(args, slab_index(), kSlab, rmask | wmask, ptr, sizeof(typename E::elem_t));
   if (n == 0) return;
   uintptr_t bits = 0;
 #pragma unroll
@@ -379,7 +389,7 @@ template <int U, bool NT>
 __global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {
   constexpr uint32_t kSlab = kThreads * 16 * U;  // bytes
   char* ptr[2];
-  const uint32_t n = TableLocator<2>::locate(args, blockIdx.x, kSlab, 3u, ptr, 1);
+  const uint32_t n = TableLocator<2>::locate(args, slab_index(), kSlab, 3u, ptr, 1);
   if (n == 0) return;
   char* dst = ptr[0];
   const char* src = ptr[1];
@@ -446,9 +456,15 @@ int check_chunk_elems(const char* what, uint32_t chunk_elems) {
   return TFT_OK;
 }
 
-// One workgroup per slab and at most 2^31-1 workgroups per grid; the smallest
-// slab any kernel uses is 1024 elements (4096 bytes for the copy kernel).
-uint32_t max_chunks(uint32_t chunk_elems) { return 0x7fffffffu / (chunk_elems / 1024u); }
+// One workgroup per slab and slab indices are 32-bit; the smallest slab any
+// kernel uses is 1024 elements (4096 bytes for the copy kernel).
+uint32_t max_chunks(uint32_t chunk_elems) { return 0xffffffffu / (chunk_elems / 1024u); }
+
+dim3 grid_for(uint64_t slabs) {
+  const uint32_t x = (uint32_t)(slabs < kMaxGridX ? slabs : kMaxGridX);
+  const uint32_t y = (uint32_t)((slabs + x - 1) / x);
+  return dim3(x, y, 1);
+}
 
 // > 0: nothing to do; < 0: error
 int check_table(const char* what, const tft_mt_table* t, uint32_t want_cols) {
@@ -481,26 +497,26 @@ int check_reduce(const char* what, uint32_t n_replicas, uint32_t mask, uint32_t 
 // slab_elems always divides chunk_elems: both are powers of two and
 // chunk_elems >= TFT_MIN_CHUNK_ELEMS >= the largest slab (256 lanes * 8 bf16 * 4;
 // 256 lanes * 16 bytes * 4 for the byte copy, whose minimum is checked there).
-TableArgs table_args(const tft_mt_table* t, uint32_t slab_elems, uint32_t* grid) {
+TableArgs table_args(const tft_mt_table* t, uint32_t slab_elems, dim3* grid) {
   const uint32_t shift = log2u(t->chunk_elems / slab_elems);
-  *grid = t->total_chunks << shift;
+  *grid = grid_for((uint64_t)t->total_chunks << shift);
   return TableArgs{static_cast<void* const*>(t->ptrs), t->numel, t->chunk_start, t->chunk_tensor,
-                   t->n_tensors, t->chunk_elems, shift};
+                   t->n_tensors, t->chunk_elems, shift, t->total_chunks};
 }
 
 template <class E, class Op, int U, bool NT>
 void launch_table(const tft_mt_table* t, const Op& op, hipStream_t stream) {
-  uint32_t grid = 0;
+  dim3 grid;
   const TableArgs a = table_args(t, kThreads * E::kVec * U, &grid);
-  hipLaunchKernelGGL((mt_stream_kernel<E, Op, TableLocator<Op::NCOL>, U, NT>), dim3(grid),
+  hipLaunchKernelGGL((mt_stream_kernel<E, Op, TableLocator<Op::NCOL>, U, NT>), grid,
                      dim3(kThreads), 0, stream, a, op);
 }
 
 template <class E, class Op, int U, bool NT>
 void launch_flat(const FlatArgs& a, const Op& op, hipStream_t stream) {
   const uint64_t slab = (uint64_t)kThreads * E::kVec * U;
-  const uint32_t grid = (uint32_t)((a.numel + slab - 1) / slab);
-  hipLaunchKernelGGL((mt_stream_kernel<E, Op, FlatLocator<Op::NCOL>, U, NT>), dim3(grid),
+  const dim3 grid = grid_for((a.numel + slab - 1) / slab);
+  hipLaunchKernelGGL((mt_stream_kernel<E, Op, FlatLocator<Op::NCOL>, U, NT>), grid,
                      dim3(kThreads), 0, stream, a, op);
 }
 
@@ -599,7 +615,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
   if (numel == 0) return TFT_OK;
   if (!out) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: out is NULL", what);
   if (n_replicas && !replicas) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: replicas is NULL", what);
-  if (numel > (1ull << 40)) return fail(TFT_ERR_UNSUPPORTED, "%s: numel too large", what);
+  if (numel > (1ull << 41)) return fail(TFT_ERR_UNSUPPORTED, "%s: numel too large", what);
   FlatArgs a{};
   a.ptrs[0] = out;
   for (uint32_t r = 0; r < n_replicas; ++r) {
@@ -712,11 +728,11 @@ int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
                 table->chunk_elems, kThreads * 16 * 4);
   const Variant v = decode_variant();
   hipStream_t s = static_cast<hipStream_t>(stream);
-  uint32_t grid = 0;
-#define TFT_COPY(UU, NTT)                                                              \
-  do {                                                                                 \
-    const TableArgs a = table_args(table, kThreads * 16 * UU, &grid);                  \
-    hipLaunchKernelGGL((mt_copy_kernel<UU, NTT>), dim3(grid), dim3(kThreads), 0, s, a); \
+  dim3 grid;
+#define TFT_COPY(UU, NTT)                                                        \
+  do {                                                                           \
+    const TableArgs a = table_args(table, kThreads * 16 * UU, &grid);            \
+    hipLaunchKernelGGL((mt_copy_kernel<UU, NTT>), grid, dim3(kThreads), 0, s, a); \
   } while (0)
   if (v.nt) {
     if (v.unroll == 4) TFT_COPY(4, true);
