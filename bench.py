@@ -82,15 +82,22 @@ class Timed:
         return wall_ms, kernel_ms
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
+# each counter scaled by its reading for a plain copy of known size; the summary is kept
+# under profiles/).  Only the headline kernel has been measured.
+MEASURED_TRAFFIC_BYTES = {"mt_stream_kernel<F32, DilocoFusedOp<2>>": 224.761e9}
+
+
 def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1) -> Dict[str, object]:
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(kernel) if algo_bytes > 2e11 else None
     return {
         "bound": "hbm",
         "achieved": achieved,
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS,
-        "traffic": None,
+        "traffic": traffic,
         "kernel": kernel,
         "kernel_ms_per_step": kernel_ms,
         "launches_per_step": launches,

@@ -171,7 +171,7 @@ int tft_mt_copy_bytes(const tft_mt_table* table, void* stream);
 
 /* Benchmark hook: selects a launch variant for later calls FROM THIS THREAD
  * (thread-local; 0 restores the tuned default).  bits 0-3: 128-bit accesses per
- * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; default 2);
+ * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; 0 = each kernel's tuned default);
  * bit 4: plain instead of non-temporal accesses. */
 void tft_set_launch_variant(uint32_t variant);
 

@@ -427,8 +427,10 @@ struct Variant {
   bool nt;
 };
 
-Variant decode_variant() {
-  Variant v{2, true};  // 8 KiB per stream and workgroup measured best on the fused step
+// default_unroll: slab size (in 4 KiB units per stream) that measured best for the
+// calling kernel on MI355X; the thread's launch variant overrides it.
+Variant decode_variant(int default_unroll) {
+  Variant v{default_unroll, true};
   const uint32_t bits = g_variant;
   if ((bits & 0xfu) == 1 || (bits & 0xfu) == 2 || (bits & 0xfu) == 4) v.unroll = (int)(bits & 0xfu);
   if (bits & 0x10u) v.nt = false;
@@ -522,9 +524,9 @@ void launch_flat(const FlatArgs& a, const Op& op, hipStream_t stream) {
 
 // Expands to the launch of LAUNCHER<E, Op, U, NT>(ARGS, op, stream) for the
 // thread's launch variant.
-#define TFT_DISPATCH_VARIANT(LAUNCHER, E, OP, ARGS, op, stream)                    \
+#define TFT_DISPATCH_VARIANT(LAUNCHER, E, OP, ARGS, op, stream, DEFAULT_U)         \
   do {                                                                             \
-    const Variant v_ = decode_variant();                                           \
+    const Variant v_ = decode_variant(DEFAULT_U);                                  \
     if (v_.nt) {                                                                   \
       if (v_.unroll == 4) LAUNCHER<E, OP, 4, true>(ARGS, op, stream);              \
       else if (v_.unroll == 2) LAUNCHER<E, OP, 2, true>(ARGS, op, stream);         \
@@ -630,9 +632,9 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
     typedef ReduceAvgOp<1, N> Op;                                              \
     const Op op{participate_mask, (float)num_participants};                    \
     if (dtype == TFT_F32)                                                      \
-      TFT_DISPATCH_VARIANT(launch_flat, F32, Op, a, op, s);                    \
+      TFT_DISPATCH_VARIANT(launch_flat, F32, Op, a, op, s, 4);                 \
     else                                                                       \
-      TFT_DISPATCH_VARIANT(launch_flat, BF16, Op, a, op, s);                   \
+      TFT_DISPATCH_VARIANT(launch_flat, BF16, Op, a, op, s, 4);                \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
@@ -655,9 +657,9 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
     typedef ReduceAvgOp<O, N> Op;                                              \
     const Op op{participate_mask, (float)num_participants};                    \
     if (dtype == TFT_F32)                                                      \
-      TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s);               \
+      TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 4);            \
     else                                                                       \
-      TFT_DISPATCH_VARIANT(launch_table, BF16, Op, table, op, s);              \
+      TFT_DISPATCH_VARIANT(launch_table, BF16, Op, table, op, s, 4);           \
   } while (0)
 #define TFT_CALL_O1(N) TFT_CALL2(1, N)
 #define TFT_CALL_O2(N) TFT_CALL2(2, N)
@@ -685,7 +687,7 @@ int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
   do {                                                                         \
     typedef DilocoFusedOp<N> Op;                                               \
     const Op op{participate_mask, (float)num_participants, k};                 \
-    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s);                 \
+    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 2);              \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
@@ -703,7 +705,7 @@ int tft_mt_pseudograd_avg_f32(const tft_mt_table* table, uint32_t n_replicas,
   do {                                                                                \
     typedef PseudogradOp<N> Op;                                                       \
     const Op op{participate_mask, (float)num_participants, restore_p ? 1u : 0u};      \
-    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s);                        \
+    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 2);                     \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
@@ -716,7 +718,7 @@ int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, v
   if (int rc = check_table(what, table, 4)) return rc < 0 ? rc : TFT_OK;
   const OuterSgdOp op{make_coef(sgd)};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  TFT_DISPATCH_VARIANT(launch_table, F32, OuterSgdOp, table, op, s);
+  TFT_DISPATCH_VARIANT(launch_table, F32, OuterSgdOp, table, op, s, 2);
   return check_launch(what);
 }
 
@@ -726,7 +728,7 @@ int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
   if (table->chunk_elems < kThreads * 16 * 4)
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: chunk_elems %u bytes is below %d", what,
                 table->chunk_elems, kThreads * 16 * 4);
-  const Variant v = decode_variant();
+  const Variant v = decode_variant(1);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid;
 #define TFT_COPY(UU, NTT)                                                        \
