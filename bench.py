@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0
 LR, MOMENTUM = 0.7, 0.9
 HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo"
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
-             "checkpoint_llama3_8b", "localsgd_llama3_8b"]
+             "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -48,9 +48,9 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=WORKLOADS, default=WORKLOADS[0])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-layers", type=int, default=2,
+    ap.add_argument("--cpu-layers", type=int, default=8,
                     help="decoder layers in the CPU baseline's slice of the Llama workload")
-    ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one plain multi-tensor copy of known size before the timed loop "
                          "(reference point for hardware-counter runs)")
@@ -123,7 +123,12 @@ def cpu_baseline_diloco(args, shapes, n_rep: int, sample: str) -> Dict[str, obje
     from oracle import replica_sync as O
     from torchft_amd import workloads
 
-    wl = workloads.make_diloco_workload(shapes, n_rep, torch.device("cpu"))
+    # draw the values on the GPU (seconds) and move them to host memory: the CPU generator
+    # needs minutes for a billion normals, and the values do not change the timing
+    wl = workloads.make_diloco_workload(shapes, n_rep, torch.device("cuda", 0))
+    wl.backup = [t.cpu() for t in wl.backup]
+    wl.replicas = [[t.cpu() for t in rep] for rep in wl.replicas]
+    torch.cuda.empty_cache()
     params = [torch.nn.Parameter(t) for t in wl.replicas[0]]
     opt = torch.optim.SGD(params, lr=LR, momentum=MOMENTUM, nesterov=True)
     pg = O.make_gloo_world1()
@@ -191,6 +196,48 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         else:
             cpu_shapes, sample = shapes, "full GPT-2-small workload"
         out["cpu_baseline"] = cpu_baseline_diloco(args, cpu_shapes, n_rep, sample)
+    return out
+
+
+def bench_diloco_api(args) -> Dict[str, object]:
+    """The same step driven through the torchft-shaped API: ``DiLoCo.sync()`` on a module
+    with the 291 Llama-3-8B parameters, this package's Manager on a local replica group of
+    2; the timed step includes all host work (quorum, commit vote, table checks)."""
+    from torch import nn
+
+    from torchft_amd import DiLoCo, Manager, ProcessGroupLocalReplicas, StaticQuorum, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+
+    class Bag(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList(
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev)])
+
+    model = Bag()
+    peer = workloads.drifted_replica([p.data for p in model.parameters()], 1e-3, 1001)
+    index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = torch.optim.SGD(model.parameters(), lr=0.1)
+    outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
+    n_params = sum(p.numel() for p in model.parameters())
+    with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
+        diloco.sync()  # first step creates the momentum state
+        wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(diloco.sync)
+    manager.shutdown(wait=False)
+    out = base_line(args, HEADLINE_METRIC + " (through DiLoCo.sync())", n_params / (wall_ms * 1e-3),
+                    "params/s", wall_ms, "f32",
+                    {"workload": "DiLoCo.sync() on a module with the 291 Llama-3-8B fp32 parameters, "
+                                 "Manager + ProcessGroupLocalReplicas(world 2), outer torch.optim.SGD "
+                                 "Nesterov; parameters updated in place (the live parameters are "
+                                 "replica 0)",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
+    out["roofline"] = roofline(n_params * 28, kernel_ms, "mt_stream_kernel<F32, DilocoFusedOp<2>>")
+    out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
     return out
 
 
@@ -325,6 +372,8 @@ def main() -> int:
         out = bench_ddp_buckets(args)
     elif args.workload == "checkpoint_llama3_8b":
         out = bench_checkpoint(args)
+    elif args.workload == "diloco_llama3_8b_api":
+        out = bench_diloco_api(args)
     else:
         out = bench_localsgd(args)
     print(json.dumps(out), flush=True)

@@ -518,3 +518,88 @@ def test_checkpoint_server_with_device_tensors(device):
     out = server.recv_checkpoint(0, server.metadata(), 8, timedelta(seconds=30))
     _assert_state_equal(out, O.state_dict_round_trip(state))
     server.shutdown()
+
+
+# ---------------------------------------------------------------------------
+# Bucketised sync through an ordinary process group (one collective per model)
+# ---------------------------------------------------------------------------
+
+class _PlainLocalPG(ProcessGroup):
+    """A process group that only offers the plain contract (``allreduce`` SUM): the flat
+    buffer it is handed is summed with a peer's flat buffer supplied by the test."""
+
+    def __init__(self, peer_flat):
+        super().__init__(0, 2)
+        self.peer_flat = peer_flat
+        self.calls = []
+
+    def configure(self, store_addr, rank, world_size):
+        pass
+
+    def allreduce(self, tensors, opts):
+        from torchft_amd import ops
+
+        for t in tensors:
+            self.calls.append(t.numel())
+            ops.reduce_avg_(t, [t, self.peer_flat(t)], 0b11, 1)
+        return _DummyWork(tensors)
+
+    def size(self):
+        return 2
+
+    def getBackendName(self):
+        return "plain-local"
+
+
+def test_diloco_bucketized_on_gpu(device):
+    torch.manual_seed(0)
+    model = MLP().to(device)
+    backup = cpu(p.data for p in model.parameters())
+    peer_params = [b + 1e-3 * torch.randn(b.shape) for b in backup]
+    # what the peer contributes to the flat buffer: its pseudo-gradients, back to back
+    peer_flat = torch.cat([(q - b).reshape(-1) for q, b in zip(peer_params, backup)]).to(device)
+    pg = _PlainLocalPG(lambda t: peer_flat)
+    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(2e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        local = cpu(p.data for p in model.parameters())
+        want = O.diloco_perform_sync([local, peer_params], backup, None, [True, True], 2, True,
+                                     lr=0.7, momentum=0.9, nesterov=True)
+        inner.step()
+        assert pg.calls == [sum(b.numel() for b in backup)]  # one collective for 6.3 M parameters
+        for p, w, m in zip(model.parameters(), want["params"], want["momentum"]):
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(outer.state[p]["momentum_buffer"], m)
+        for b, w in zip(diloco._backup_parameters.values(), want["backup"]):
+            assert_bits_equal(b, w)
+    manager.shutdown(wait=False)
+
+
+def test_local_sgd_bucketized_on_gpu(device):
+    torch.manual_seed(0)
+    model = MLP().to(device)
+    peer_params = [p.data.cpu() + 1e-3 * torch.randn(p.shape) for p in model.parameters()]
+    peer_flat = torch.cat([q.reshape(-1) for q in peer_params]).to(device)
+    pg = _PlainLocalPG(lambda t: peer_flat)
+    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
+        backup = cpu(lsgd._backup_parameters.values())
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(2e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        local = cpu(p.data for p in model.parameters())
+        want = O.localsgd_perform_sync([local, peer_params], backup, [True, True], 2, True)
+        optimizer.step()
+        assert pg.calls == [sum(b.numel() for b in backup)]
+        for p, w in zip(model.parameters(), want["params"]):
+            assert_bits_equal(p.data, w)
+        for b, w in zip(lsgd._backup_parameters.values(), want["backup"]):
+            assert_bits_equal(b, w)
+    manager.shutdown(wait=False)

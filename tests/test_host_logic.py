@@ -492,12 +492,11 @@ def test_diloco_fused_on_local_replicas(cpu_ops, commit):
                 for q, b in zip(peer.parameters(), backup):
                     q.data.copy_(b + 1e-3 * (k + 1) * torch.randn_like(b))
             cpu_ops.calls.clear()
-            inner.zero_grad()
-            model(torch.rand(2, 3)).mean().backward()
-            before = [p.data.clone() for p in model.parameters()]
-            # what the sync must produce, from the state just before inner.step() syncs
-            grads = [p.grad.clone() for p in model.parameters()]
-            local = [b_ - 0.1 * g for b_, g in zip(before, grads)]
+            with torch.no_grad():  # an exact local drift; inner.step() is then a no-op
+                for p in model.parameters():
+                    p.add_(1e-3 * torch.randn_like(p))
+                    p.grad = torch.zeros_like(p)
+            local = [p.data.clone() for p in model.parameters()]
             want = O.diloco_perform_sync(
                 [local] + [[q.data.clone() for q in peer.parameters()] for peer in peers],
                 backup, bufs, [True] * 3, 3, commit, lr=0.7, momentum=0.9, nesterov=True)
@@ -531,8 +530,11 @@ def test_local_sgd_fused_on_local_replicas(cpu_ops):
                       quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=0.1)
     with LocalSGD(manager, model, optimizer, sync_every=1) as local_sgd:
-        model(torch.rand(2, 3)).mean().backward()
-        local = [p.data - 0.1 * p.grad for p in model.parameters()]
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        local = [p.data.clone() for p in model.parameters()]
         want = O.localsgd_perform_sync(
             [local, [q.data.clone() for q in peers[0].parameters()]],
             [b.clone() for b in local_sgd._backup_parameters.values()], [True, True], 2, True)
@@ -678,3 +680,81 @@ def test_kernels_refuse_cpu_tensors():
         model(torch.rand(2, 3)).mean().backward()
         with pytest.raises(RuntimeError, match="no CPU path"):
             inner.step()
+
+
+# ---------------------------------------------------------------------------
+# Bucketised sync through an ordinary process group
+# ---------------------------------------------------------------------------
+
+class _DoublingPG(ProcessGroup):
+    """A fake 2-replica backend: the peer's contribution equals ours, so SUM doubles."""
+
+    def __init__(self):
+        super().__init__(0, 2)
+        self.calls = []
+
+    def configure(self, store_addr, rank, world_size):
+        pass
+
+    def allreduce(self, tensors, opts):
+        self.calls.append([t.numel() for t in tensors])
+        for t in tensors:
+            t.mul_(2)
+        return _DummyWork(tensors)
+
+    def size(self):
+        return 2
+
+    def getBackendName(self):
+        return "doubling"
+
+
+def test_diloco_bucketized_one_collective_per_sync(cpu_ops):
+    torch.manual_seed(0)
+    model = SimpleModel()
+    pg = _DoublingPG()
+    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    backup = [p.data.clone() for p in model.parameters()]
+    n_total = sum(p.numel() for p in model.parameters())
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        with torch.no_grad():  # an exact local drift; the inner step itself is then a no-op
+            for p in model.parameters():
+                p.add_(1e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        local = [p.data.clone() for p in model.parameters()]
+        # both replicas hold the same parameters => the average equals the local pseudo-gradient
+        want = O.diloco_perform_sync([local, local], backup, None, [True, True], 2, True,
+                                     lr=0.7, momentum=0.9, nesterov=True)
+        inner.step()
+        assert pg.calls == [[n_total]]  # the whole model in one collective
+        for p, w in zip(model.parameters(), want["params"]):
+            assert_bits_equal(p.data, w)
+        for b, w in zip(diloco._backup_parameters.values(), want["backup"]):
+            assert_bits_equal(b, w)
+        assert cpu_ops.calls.count("mt_pseudograd_avg") == 1 and cpu_ops.calls.count("mt_outer_sgd") == 1
+    manager.shutdown(wait=False)
+
+
+def test_local_sgd_bucketized_one_collective_per_sync(cpu_ops):
+    torch.manual_seed(0)
+    model = SimpleModel()
+    pg = _DoublingPG()
+    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    n_total = sum(p.numel() for p in model.parameters())
+    with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        local = [p.data.clone() for p in model.parameters()]
+        optimizer.step()
+        assert pg.calls == [[n_total]]
+        for p, w in zip(model.parameters(), local):
+            assert_bits_equal(p.data, w)  # (x + x) / 2 == x exactly
+        torch.testing.assert_close(lsgd._backup_parameters, _params_dict(model))
+    manager.shutdown(wait=False)

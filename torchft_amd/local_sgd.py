@@ -16,6 +16,12 @@ Manager and commits or rolls back.  What differs is how the work is issued:
   DMA copies); DiLoCo needs the backup on the device, as the reference's
   ``p.data - backup`` does for GPU parameters.
 
+With this package's Manager on any other process group (one real collective per call) the
+model is bucketised: the pseudo-gradients (DiLoCo) or a flattened copy of the weights
+(LocalSGD) live in ONE flat buffer per dtype and a single ``manager.allreduce`` covers the
+whole model, instead of the reference's one collective per parameter
+(``torchft/local_sgd.py:170`` "TODO: bucketize parameters").
+
 With a Manager that is not this package's (for instance a mock) the per-parameter
 ``manager.allreduce`` contract is kept call for call.
 """
@@ -72,6 +78,7 @@ class LocalSGD:
             self._backup_parameters[name] = t
         self._hooks: List[RemovableHandle] = []
         self._tables: Dict[str, TensorTable] = {}
+        self._flat: Dict[str, tuple] = {}
         # the first sync needs a valid backup
         self._save_parameters()
 
@@ -126,6 +133,26 @@ class LocalSGD:
         for d, s in zip(dsts, srcs):  # host-resident backup: plain DMA, no arithmetic
             d.copy_(s, non_blocking=not blocking)
 
+    def _flat_like(self, key: str, tensors: Sequence[torch.Tensor]):
+        """One flat buffer per dtype with the sizes of ``tensors`` back to back, plus a view
+        per tensor (in the order of ``tensors``).  Kept across syncs."""
+        cached = self._flat.get(key)
+        sig = tuple((t.dtype, t.device, tuple(t.shape)) for t in tensors)
+        if cached is not None and cached[0] == sig:
+            return cached[1], cached[2]
+        flats: Dict[torch.dtype, torch.Tensor] = {}
+        for dtype in {t.dtype for t in tensors}:
+            n = sum(t.numel() for t in tensors if t.dtype == dtype)
+            flats[dtype] = torch.empty(n, dtype=dtype, device=tensors[0].device)
+        offsets = {dtype: 0 for dtype in flats}
+        views = []
+        for t in tensors:
+            off = offsets[t.dtype]
+            views.append(flats[t.dtype][off : off + t.numel()].view(t.shape))
+            offsets[t.dtype] = off + t.numel()
+        self._flat[key] = (sig, flats, views)
+        return flats, views
+
     def _save_parameters(self) -> None:
         """backup <- parameters (torchft/local_sgd.py:121-125), one launch."""
         with torch.no_grad():
@@ -167,12 +194,24 @@ class LocalSGD:
                     self._restore_parameters()
                 return
             self._manager.allreduce_tensors(params).wait()
+        elif _is_native_manager(self._manager) and self._on_device(params, backups):
+            self._average_bucketized(params)
         else:
             self._average()
         if self._manager.should_commit():
             self._save_parameters()
         else:
             self._restore_parameters()
+
+    def _average_bucketized(self, params: List[torch.Tensor]) -> None:
+        """Flatten (one launch), ONE ``manager.allreduce`` per dtype, unflatten (one launch)."""
+        flats, views = self._flat_like("weights", params)
+        self._tables["flatten"] = ops.mt_copy(views, params, table=self._tables.get("flatten"))
+        works = [self._manager.allreduce(flat) for flat in flats.values()]
+        for work in works:
+            work.wait()
+        if self._manager.errored() is None:
+            self._tables["unflatten"] = ops.mt_copy(params, views, table=self._tables.get("unflatten"))
 
     def _average(self) -> None:
         works = []
@@ -319,7 +358,8 @@ class DiLoCo(LocalSGD):
             self._outer_optimizer.zero_grad()
             return
 
-        grads = self._grad_buffers(params)
+        bucketized = not fused and _is_native_manager(self._manager)
+        grads = self._flat_like("grads", params)[1] if bucketized else self._grad_buffers(params)
         if fused:
             # pseudo-gradient, replica sum, divide and restore: one launch
             for p, g in zip(live, grads):
@@ -327,6 +367,18 @@ class DiLoCo(LocalSGD):
             self._manager.pseudograd_allreduce(grads, params, backups, restore_params=True).wait()
             if self._manager.errored() is not None:
                 self._restore_parameters()  # the launch that restores did not happen
+        elif bucketized:
+            # pseudo-gradients written straight into one flat buffer (and the parameters
+            # restored) by one launch, then ONE collective for the whole model
+            self._tables["pseudograd"] = ops.mt_pseudograd_avg(
+                grads, params, backups, [params], restore_params=True,
+                table=self._tables.get("pseudograd"),
+            )
+            for p, g in zip(live, grads):
+                p.grad = g
+            works = [self._manager.allreduce(flat) for flat in self._flat_like("grads", params)[0].values()]
+            for work in works:
+                work.wait()
         else:
             # pseudo-gradients in one launch, then the Manager contract per parameter
             self._tables["pseudograd"] = ops.mt_pseudograd_avg(
