@@ -170,13 +170,34 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         ops.mt_copy(params, wl.backup)
         torch.cuda.synchronize()
 
+    # The reference computes the pseudo-gradient as params - backup and lets SGD subtract it
+    # (torchft/local_sgd.py:214, :223), so with replicas that never move the backup runs away
+    # from them geometrically and overflows fp32 after about 95 applications.  Real training
+    # restarts the replicas from the new backup after every sync; a benchmark with static
+    # inputs instead puts the pristine backup and momentum back every RESEED steps (two
+    # multi-tensor copies, counted inside the timed region).  Runs of up to RESEED steps in
+    # total (the default) never re-seed.
+    RESEED = 64
+    need_reseed = args.steps + args.warmup > RESEED
+    pristine = None
+    if need_reseed:
+        pristine = ([t.clone() for t in wl.backup], [t.clone() for t in bufs])
+    done = [0]
+    reseeds = [0]
+
     def step() -> None:
+        if pristine is not None and done[0] and done[0] % RESEED == 0:
+            ops.mt_copy(wl.backup, pristine[0])
+            ops.mt_copy(bufs, pristine[1])
+            reseeds[0] += 1
         ops.mt_diloco_outer(params, wl.backup, bufs, wl.replicas, sgd, False, table=table)
+        done[0] += 1
 
     wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
-    probe = len(params) // 2
-    if not torch.isfinite(params[probe]).all() or not torch.equal(params[probe], wl.backup[probe]):
-        raise RuntimeError("output check failed: parameters are not finite or differ from the backup")
+    for probe in (0, len(params) // 2, len(params) - 1):
+        same = torch.equal(params[probe].view(torch.int32), wl.backup[probe].view(torch.int32))
+        if not same or not torch.isfinite(params[probe]).all():
+            raise RuntimeError("output check failed: parameters are not finite or differ from the backup")
 
     n_params = wl.n_params
     # read N replicas, backup, momentum; write momentum, parameters, backup
@@ -189,6 +210,10 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
                      f"momentum={MOMENTUM}, one fused multi-tensor launch per step",
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
     out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>")
+    if reseeds[0]:
+        out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]
+        out["roofline"]["note"] = ("steps that re-seed the state include two extra copy launches in "
+                                   "kernel_ms_per_step")
     if not args.no_cpu_baseline:
         if which == "llama3_8b":
             cpu_shapes = workloads.llama3_8b_shapes(args.cpu_layers, with_embeddings=False)
@@ -225,6 +250,9 @@ def bench_diloco_api(args) -> Dict[str, object]:
     inner = torch.optim.SGD(model.parameters(), lr=0.1)
     outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
     n_params = sum(p.numel() for p in model.parameters())
+    if args.steps + args.warmup > 60:
+        raise SystemExit("diloco_llama3_8b_api: at most 60 syncs in total (static peers make the "
+                         "backup run away from them; see bench_diloco)")
     with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
         diloco.sync()  # first step creates the momentum state
         wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(diloco.sync)
