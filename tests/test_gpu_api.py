@@ -603,3 +603,57 @@ def test_local_sgd_bucketized_on_gpu(device):
         for b, w in zip(lsgd._backup_parameters.values(), want["backup"]):
             assert_bits_equal(b, w)
     manager.shutdown(wait=False)
+
+
+# ---------------------------------------------------------------------------
+# Host-resident backup (the reference's default placement), moved as one transfer
+# ---------------------------------------------------------------------------
+
+def test_localsgd_host_backup_one_transfer(device):
+    torch.manual_seed(0)
+    model = MLP().to(device)
+    manager = create_autospec(Manager)
+    manager.should_commit.return_value = True
+    manager.allreduce.side_effect = lambda t: _done(t)
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1, backup_device=torch.device("cpu")) as lsgd:
+        for name, b in lsgd._backup_parameters.items():
+            assert b.device.type == "cpu" and b.is_pinned(), name
+        lsgd._host_backup.wait()
+        for (name, p), b in zip(model.named_parameters(), lsgd._backup_parameters.values()):
+            assert_bits_equal(b, p.data, f"initial backup {name}")
+        before = cpu(p.data for p in model.parameters())
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1.0)
+        lsgd._restore_parameters()  # local changes discarded
+        for p, w in zip(model.parameters(), before):
+            assert_bits_equal(p.data, w)
+        # a committed sync refreshes the host copy (asynchronously; wait before reading it)
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(0.5)
+                p.grad = torch.zeros_like(p)
+        optimizer.step()
+        lsgd._host_backup.wait()
+        for (name, p), b in zip(model.named_parameters(), lsgd._backup_parameters.values()):
+            assert_bits_equal(b, p.data, f"backup after commit {name}")
+        # refused commit: parameters come back from the host copy
+        manager.should_commit.return_value = False
+        want = cpu(p.data for p in model.parameters())
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(0.25)
+        optimizer.step()
+        for p, w in zip(model.parameters(), want):
+            assert_bits_equal(p.data, w)
+        # a user may replace the backup tensors (torchft/manager_integ_test.py:279)
+        lsgd._backup_parameters = {n: torch.zeros_like(b) for n, b in lsgd._backup_parameters.items()}
+        lsgd._restore_parameters()
+        assert all(int(torch.count_nonzero(p.data)) == 0 for p in model.parameters())
+
+
+def _done(t):
+    f = Future()
+    f.set_result(t)
+    return f

@@ -758,3 +758,32 @@ def test_local_sgd_bucketized_one_collective_per_sync(cpu_ops):
             assert_bits_equal(p.data, w)  # (x + x) / 2 == x exactly
         torch.testing.assert_close(lsgd._backup_parameters, _params_dict(model))
     manager.shutdown(wait=False)
+
+
+def test_manager_client_adapter(cpu_ops):
+    """A client with the reference's ManagerClient signatures (torchft/torchft.pyi:4-23),
+    mocked the way torchft/manager_test.py patches it, drives this package's Manager."""
+    from torchft_amd import ManagerClientAdapter
+
+    client = MagicMock()
+    client.quorum.return_value = QuorumResult(quorum_id=123, replica_rank=1, replica_world_size=2,
+                                              max_step=1, max_rank=1, max_world_size=2)
+    client.should_commit.side_effect = lambda rank, step, should_commit, timeout: should_commit
+    peer = MagicMock()
+    peer.checkpoint_metadata.return_value = "http://peer/checkpoint/"
+    adapter = ManagerClientAdapter(client, connect=lambda address: peer)
+    m = Manager(pg=create_autospec(ProcessGroup), min_replica_size=2, quorum_client=adapter,
+                timeout=timedelta(seconds=7))
+    m._pg.allreduce.return_value = _DummyWork(None)
+    m.start_quorum(timeout=timedelta(seconds=12))
+    m.wait_quorum()
+    assert client.quorum.call_args.kwargs["timeout"] == timedelta(seconds=12)  # manager_test.py:560-563
+    assert client.quorum.call_args.kwargs["rank"] == 0 and client.quorum.call_args.kwargs["step"] == 0
+    t = torch.tensor([2.0])
+    m.allreduce(t).wait()
+    torch.testing.assert_close(t, torch.tensor([1.0]))
+    assert m.should_commit(timeout=timedelta(seconds=23))
+    assert client.should_commit.call_args.kwargs["timeout"] == timedelta(seconds=23)
+    assert adapter.checkpoint_metadata("addr", 3, timedelta(seconds=1)) == "http://peer/checkpoint/"
+    peer.checkpoint_metadata.assert_called_once_with(3, timeout=timedelta(seconds=1))
+    m.shutdown(wait=False)

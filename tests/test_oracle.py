@@ -280,7 +280,7 @@ def test_bucket_assignment_is_torchs(shapes_fn, dtype):
     assert got == want
 
 
-def test_bucket_assignment_llama_matches_torch_and_survey_count():
+def test_bucket_assignment_llama_matches_torch_and_known_count():
     shapes = workloads.llama3_8b_shapes()
     metas = [torch.empty(s, dtype=torch.bfloat16, device="meta") for _, s in shapes]
     want = _torch_bucket_assignment(metas, O.DEFAULT_FIRST_BUCKET_BYTES, O.DEFAULT_BUCKET_CAP_BYTES)
@@ -322,7 +322,7 @@ def test_bucket_layout_against_a_real_reducer():
         assert members == buckets[index]
         assert offsets == O.bucket_offsets(numels, buckets[index])
         assert total == sum(numels[i] for i in members)
-    # the sizes the survey of the reference recorded for this model
+    # the bucket sizes torch produces for this model (4 218 890 and 2 097 152 elements)
     assert sorted(s[3] for s in seen) == [2_097_152, 4_218_890]
 
 

@@ -10,7 +10,14 @@ declared in ``include/torchft_amd.h``; there is no CPU fallback.
 from .checkpointing import CheckpointServer, CheckpointTransport
 from .ddp import DistributedDataParallel, GradBucketAverager, PureDistributedDataParallel
 from .local_sgd import DiLoCo, LocalSGD
-from .manager import Manager, QuorumClient, QuorumResult, StaticQuorum, WorldSizeMode
+from .manager import (
+    Manager,
+    ManagerClientAdapter,
+    QuorumClient,
+    QuorumResult,
+    StaticQuorum,
+    WorldSizeMode,
+)
 from .optim import OptimizerWrapper as Optimizer
 from .optim import OptimizerWrapper
 from .process_group import (
@@ -27,6 +34,7 @@ __all__ = (
     "GradBucketAverager",
     "LocalSGD",
     "Manager",
+    "ManagerClientAdapter",
     "Optimizer",
     "OptimizerWrapper",
     "ProcessGroup",

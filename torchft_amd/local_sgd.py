@@ -36,7 +36,7 @@ import torch
 from torch import nn, optim
 from torch.utils.hooks import RemovableHandle
 
-from . import ops
+from . import _native, ops
 from .manager import Manager
 from .multi_tensor import TensorTable
 
@@ -46,6 +46,71 @@ logger: logging.Logger = logging.getLogger(__name__)
 def _is_native_manager(manager: object) -> bool:
     # a create_autospec(Manager) double passes isinstance() but is not a subclass instance
     return issubclass(type(manager), Manager)
+
+
+class _PackedHostBackup:
+    """Backup of GPU parameters in pinned host memory, moved as ONE transfer.
+
+    The reference copies tensor by tensor into pinned host tensors on the compute
+    stream (torchft/local_sgd.py:121-131, with a TODO to use a separate stream).  Here
+    the parameters are gathered into a device staging buffer by one launch and the
+    staging buffer crosses PCIe as a single copy on a side stream, so the save overlaps
+    the next inner steps; restore is the same path backwards.  The tensors handed out
+    as ``_backup_parameters`` are views into the one pinned buffer.
+    """
+
+    ALIGN = 256
+
+    def __init__(self, named_params, pin_memory: bool) -> None:
+        params = [p for _, p in named_params]
+        self.device = params[0].device
+        offsets, off = [], 0
+        for p in params:
+            offsets.append(off)
+            off += -(-(p.numel() * p.element_size()) // self.ALIGN) * self.ALIGN
+        self.total = max(off, self.ALIGN)
+        self.host = torch.empty(self.total, dtype=torch.uint8, pin_memory=pin_memory)
+        self.staging = torch.empty(self.total, dtype=torch.uint8, device=self.device)
+        self.host_views = [
+            self.host[o : o + p.numel() * p.element_size()].view(p.dtype).view(p.shape)
+            for o, p in zip(offsets, params)
+        ]
+        self.staging_views = [
+            self.staging[o : o + p.numel() * p.element_size()] for o, p in zip(offsets, params)
+        ]
+        self.stream = torch.cuda.Stream(device=self.device)
+        self.host_ready: Optional[torch.cuda.Event] = None  # the last save has reached the host
+        self._tables: Dict[str, TensorTable] = {}
+
+    def owns(self, backups: Sequence[torch.Tensor]) -> bool:
+        return len(backups) == len(self.host_views) and all(
+            b.data_ptr() == v.data_ptr() for b, v in zip(backups, self.host_views)
+        )
+
+    def save(self, params: List[torch.Tensor]) -> None:
+        current = torch.cuda.current_stream(self.device)
+        if self.host_ready is not None:
+            current.wait_event(self.host_ready)  # staging is free again
+        self._tables["pack"] = ops.mt_copy(self.staging_views, params, table=self._tables.get("pack"))
+        packed = torch.cuda.Event()
+        packed.record(current)
+        self.stream.wait_event(packed)
+        with torch.cuda.stream(self.stream):
+            self.host.copy_(self.staging, non_blocking=True)
+            self.host_ready = torch.cuda.Event()
+            self.host_ready.record(self.stream)
+
+    def wait(self) -> None:
+        """Blocks until the host copy is complete (before anything reads the backup)."""
+        if self.host_ready is not None:
+            self.host_ready.synchronize()
+
+    def restore(self, params: List[torch.Tensor]) -> None:
+        self.wait()
+        current = torch.cuda.current_stream(self.device)
+        self.staging.copy_(self.host, non_blocking=True)
+        self._tables["unpack"] = ops.mt_copy(params, self.staging_views, table=self._tables.get("unpack"))
+        current.synchronize()  # the reference's restore is blocking
 
 
 class LocalSGD:
@@ -70,12 +135,27 @@ class LocalSGD:
         self._sync_every = sync_every
         assert sync_every >= 1, "sync_every must be greater than or equal to 1"
         self._backup_parameters: Dict[str, torch.Tensor] = {}
-        for name, p in self._model.named_parameters():
-            device = backup_device if backup_device is not None else p.device
-            t = torch.empty(*tuple(p.shape), dtype=p.dtype, device=device)
-            if pin_memory and t.device == torch.device("cpu") and torch.cuda.is_available():
-                t = t.pin_memory()
-            self._backup_parameters[name] = t
+        self._host_backup: Optional[_PackedHostBackup] = None
+        named = list(self._model.named_parameters())
+        if (
+            backup_device is not None
+            and torch.device(backup_device).type == "cpu"
+            and named
+            and all(p.is_cuda and p.device == named[0][1].device for _, p in named)
+        ):
+            # GPU parameters with a host backup: one pinned buffer, one transfer per save
+            self._host_backup = _PackedHostBackup(named, pin_memory)
+            for (name, _), view in zip(named, self._host_backup.host_views):
+                self._backup_parameters[name] = view
+        else:
+            for name, p in named:
+                device = backup_device if backup_device is not None else p.device
+                t = torch.empty(*tuple(p.shape), dtype=p.dtype, device=device)
+                if pin_memory and t.device == torch.device("cpu") and torch.cuda.is_available():
+                    t = t.pin_memory()
+                self._backup_parameters[name] = t
+        if named and any(p.is_cuda for _, p in named):
+            _native.lib()  # GPU parameters need the kernels: fail now, loudly, if they are missing
         self._hooks: List[RemovableHandle] = []
         self._tables: Dict[str, TensorTable] = {}
         self._flat: Dict[str, tuple] = {}
@@ -157,12 +237,20 @@ class LocalSGD:
         """backup <- parameters (torchft/local_sgd.py:121-125), one launch."""
         with torch.no_grad():
             _, params, backups = self._named()
+            if self._host_backup is not None and self._host_backup.owns(backups):
+                self._host_backup.save(params)
+                return
             self._copy("save", backups, params, blocking=False)
 
     def _restore_parameters(self) -> None:
         """parameters <- backup (torchft/local_sgd.py:127-131), one launch."""
         with torch.no_grad():
             _, params, backups = self._named()
+            if self._host_backup is not None:
+                if self._host_backup.owns(backups):
+                    self._host_backup.restore(params)
+                    return
+                self._host_backup.wait()  # the user swapped the backup tensors: plain copies
             self._copy("restore", params, backups, blocking=True)
 
     # -- sync ------------------------------------------------------------------

@@ -117,6 +117,32 @@ class StaticQuorum(QuorumClient):
         return should_commit
 
 
+class ManagerClientAdapter(QuorumClient):
+    """Puts a client with the reference's ``ManagerClient`` interface
+    (torchft/torchft.pyi:4-23: ``quorum``, ``should_commit``, ``checkpoint_metadata(rank,
+    timeout)``) into the ``QuorumClient`` seat.  ``connect(address)`` must return such a
+    client for another replica group's manager (torchft: ``ManagerClient(address,
+    connect_timeout=...)``, torchft/manager.py:497-502)."""
+
+    def __init__(self, client: object, connect: Optional[Callable[[str], object]] = None) -> None:
+        self._client = client
+        self._connect = connect
+
+    def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+        return self._client.quorum(
+            rank=rank, step=step, checkpoint_metadata=checkpoint_metadata,
+            shrink_only=shrink_only, timeout=timeout,
+        )
+
+    def should_commit(self, rank, step, should_commit, timeout):
+        return self._client.should_commit(rank, step, should_commit, timeout=timeout)
+
+    def checkpoint_metadata(self, address, rank, timeout):
+        if self._connect is None:
+            raise NotImplementedError("no way to connect to other managers was given")
+        return self._connect(address).checkpoint_metadata(rank, timeout=timeout)
+
+
 def _done_future(value: object) -> torch.futures.Future:
     fut: torch.futures.Future = torch.futures.Future()
     fut.set_result(value)
