@@ -41,8 +41,8 @@
  *     not read;
  *   - the sum is divided (IEEE divide, not reciprocal multiply) by
  *     num_participants, which may differ from popcount(participate_mask);
- *   - bf16 inputs are widened to fp32, accumulated and divided in fp32, and
- *     rounded to nearest-even once on store.
+ *   - bf16 and fp16 inputs are widened to fp32, accumulated and divided in fp32,
+ *     and rounded to nearest-even once on store.
  */
 #ifndef TORCHFT_AMD_H_
 #define TORCHFT_AMD_H_
@@ -53,7 +53,7 @@
 extern "C" {
 #endif
 
-#define TFT_ABI_VERSION 2
+#define TFT_ABI_VERSION 3
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
 #define TFT_MIN_CHUNK_ELEMS 8192u
 
@@ -64,7 +64,7 @@ typedef enum tft_status {
   TFT_ERR_LAUNCH = -3
 } tft_status;
 
-typedef enum tft_dtype { TFT_F32 = 0, TFT_BF16 = 1 } tft_dtype;
+typedef enum tft_dtype { TFT_F32 = 0, TFT_BF16 = 1, TFT_F16 = 2 } tft_dtype;
 
 /* Host struct describing one multi-tensor table (the arrays live on the device). */
 typedef struct tft_mt_table {

@@ -29,7 +29,7 @@ def draw(n, dtype, seed, scale=1.0):
     return (torch.randn(n, generator=g) * scale).to(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n_replicas,mask,nump", [
     (1, 0b1, 1), (1, 0b1, 5), (1, 0b0, 5), (2, 0b11, 2), (3, 0b101, 2), (4, 0b1011, 3),
     (4, 0b1111, 4), (8, 0xFF, 8), (8, 0b10110101, 2), (0, 0, 3),
@@ -46,7 +46,7 @@ def test_reduce_avg_flat(device, dtype, n_replicas, mask, nump):
         assert_bits_equal(out, want, f"numel={numel}")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_reduce_avg_in_place_and_misaligned(device, dtype):
     # out aliases replica 1; all buffers start 1 element past a 16-byte boundary
     numel = 70_001
@@ -86,7 +86,7 @@ def _mlp_workload(n_replicas, seed_shift=0):
     return wl
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n_outs", [1, 2])
 def test_mt_reduce_avg(device, dtype, n_outs):
     wl = _mlp_workload(3)
@@ -234,6 +234,21 @@ def test_launch_variants_agree(device):
                 assert_bits_equal(m[i], want["momentum"][i], f"variant {unroll}/{plain} {name}")
     finally:
         ops.set_launch_variant(0)
+
+
+def test_fp16_rounding_and_overflow(device):
+    """fp16 goes through fp32: one rounding to nearest even, overflow to inf, NaN stays NaN."""
+    vals = [65504.0, 65504.0, 1.0, 1.0009765625, float("nan"), 6.0e-8, -0.0]
+    a = torch.tensor(vals, dtype=torch.float16)
+    b = torch.tensor([65504.0, -65504.0, 1.0009765625, 1.0009765625, 1.0, 6.0e-8, 0.0], dtype=torch.float16)
+    want = O.manager_allreduce_([a, b], [True, True], 1, torch.float32)
+    out = torch.empty_like(a).to(device)
+    ops.reduce_avg_(out, [a.to(device), b.to(device)], 0b11, 1)
+    out = out.cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out), nan)  # the NaN payload is not part of the contract
+    assert_bits_equal(out[~nan], want[~nan])
+    assert torch.isinf(out[0]) and float(out[1]) == 0.0 and torch.isnan(out[4])
 
 
 def test_argument_errors(device):

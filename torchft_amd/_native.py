@@ -18,13 +18,14 @@ import torch  # noqa: F401  (must precede loading the library, see module docstr
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchft_amd.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 MAX_REPLICAS = 8
 MIN_CHUNK_ELEMS = 8192
 MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
 
 TFT_F32 = 0
 TFT_BF16 = 1
+TFT_F16 = 2
 
 
 class MtTable(Structure):

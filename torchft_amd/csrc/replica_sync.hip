@@ -17,6 +17,7 @@
 // Entry points are declared and documented in include/torchft_amd.h.
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
@@ -90,6 +91,29 @@ struct BF16 {
   }
   __device__ static inline float widen1(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
   __device__ static inline uint16_t narrow1(float x) { return (uint16_t)f32_to_bf16_bits(x); }
+};
+
+struct F16 {
+  typedef uint16_t elem_t;
+  static constexpr int kVec = 8;
+  __device__ static inline float widen1(uint16_t x) { return __half2float(__ushort_as_half(x)); }
+  __device__ static inline uint16_t narrow1(float x) {
+    return __half_as_ushort(__float2half_rn(x));  // round to nearest even
+  }
+  __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = widen1((uint16_t)(raw[i] & 0xffffu));
+      v[2 * i + 1] = widen1((uint16_t)(raw[i] >> 16));
+    }
+  }
+  __device__ static inline u32x4 narrow(const float (&v)[kVec]) {
+    u32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      raw[i] = (uint32_t)narrow1(v[2 * i]) | ((uint32_t)narrow1(v[2 * i + 1]) << 16);
+    return raw;
+  }
 };
 
 template <bool NT>
@@ -626,7 +650,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
                    int dtype, void* stream) {
   static const char* what = "tft_reduce_avg";
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (dtype != TFT_F32 && dtype != TFT_BF16)
+  if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
     return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
   if (numel == 0) return TFT_OK;
   if (!out) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: out is NULL", what);
@@ -647,8 +671,10 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
     const Op op{participate_mask, (float)num_participants};                    \
     if (dtype == TFT_F32)                                                      \
       TFT_DISPATCH_VARIANT(launch_flat, F32, Op, a, op, s, 4);                 \
-    else                                                                       \
+    else if (dtype == TFT_BF16)                                                \
       TFT_DISPATCH_VARIANT(launch_flat, BF16, Op, a, op, s, 4);                \
+    else                                                                       \
+      TFT_DISPATCH_VARIANT(launch_flat, F16, Op, a, op, s, 4);                 \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
@@ -662,7 +688,7 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
   if (n_outs != 1 && n_outs != 2)
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: n_outs must be 1 or 2, got %u", what, n_outs);
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (dtype != TFT_F32 && dtype != TFT_BF16)
+  if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
     return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
   if (int rc = check_table(what, table, n_outs + n_replicas)) return rc < 0 ? rc : TFT_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -672,8 +698,10 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
     const Op op{participate_mask, (float)num_participants};                    \
     if (dtype == TFT_F32)                                                      \
       TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 4);            \
-    else                                                                       \
+    else if (dtype == TFT_BF16)                                                \
       TFT_DISPATCH_VARIANT(launch_table, BF16, Op, table, op, s, 4);           \
+    else                                                                       \
+      TFT_DISPATCH_VARIANT(launch_table, F16, Op, table, op, s, 4);            \
   } while (0)
 #define TFT_CALL_O1(N) TFT_CALL2(1, N)
 #define TFT_CALL_O2(N) TFT_CALL2(2, N)

@@ -17,7 +17,11 @@ import torch
 
 from . import _native
 
-_DTYPE_CODES = {torch.float32: _native.TFT_F32, torch.bfloat16: _native.TFT_BF16}
+_DTYPE_CODES = {
+    torch.float32: _native.TFT_F32,
+    torch.bfloat16: _native.TFT_BF16,
+    torch.float16: _native.TFT_F16,
+}
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -25,7 +29,7 @@ def dtype_code(dtype: torch.dtype) -> int:
         return _DTYPE_CODES[dtype]
     except KeyError:
         raise TypeError(
-            f"torchft_amd kernels support float32 and bfloat16, got {dtype}"
+            f"torchft_amd kernels support float32, bfloat16 and float16, got {dtype}"
         ) from None
 
 
