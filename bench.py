@@ -85,7 +85,7 @@ class Timed:
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
 # each counter scaled by its reading for a plain copy of known size; the summary is kept
 # under profiles/).  Only the headline kernel has been measured.
-MEASURED_TRAFFIC_BYTES = {"mt_stream_kernel<F32, DilocoFusedOp<2>>": 224.761e9}
+MEASURED_TRAFFIC_BYTES = {"mt_stream_kernel<F32, DilocoFusedOp<2>>": 224.810e9}
 
 
 def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1) -> Dict[str, object]:
