@@ -72,6 +72,17 @@ def _timed_acquire(lock: threading.Lock, timeout: timedelta) -> Generator[None, 
         lock.release()
 
 
+def _advertised_host() -> str:
+    """The host name peers should use (as in the reference, torchft/checkpointing.py:214-216),
+    or ``localhost`` when this machine's own name does not resolve (bare containers)."""
+    host = socket.gethostname()
+    try:
+        socket.getaddrinfo(host, None)
+        return host
+    except OSError:
+        return "localhost"
+
+
 class _IPv6HTTPServer(ThreadingHTTPServer):
     address_family = socket.AF_INET6
     request_queue_size = 1024
@@ -177,7 +188,7 @@ class CheckpointServer(CheckpointTransport[T]):
     def address(self) -> str:
         """``http://host:port/checkpoint/``; the step number is appended by the fetcher."""
         port = self._server.socket.getsockname()[1]
-        return f"http://{socket.gethostname()}:{port}/checkpoint/"
+        return f"http://{_advertised_host()}:{port}/checkpoint/"
 
     # -- gate ------------------------------------------------------------------
     def disallow_checkpoint(self) -> None:
