@@ -1,0 +1,211 @@
+"""Several replica groups as threads of one process, with failure injection and restart:
+the harness of the reference's integration tests (torchft/manager_integ_test.py:39-250),
+on this package's in-process lighthouse, thread process group and checkpoint server."""
+
+import copy
+import threading
+from concurrent.futures import ThreadPoolExecutor, as_completed
+from datetime import timedelta
+from typing import Callable, Dict, List, Optional
+
+import torch
+from torch import nn, optim
+
+from torchft_amd import (
+    CheckpointServer,
+    DiLoCo,
+    DistributedDataParallel,
+    InProcessLighthouse,
+    LocalSGD,
+    Manager,
+    OptimizerWrapper,
+    ProcessGroupThreads,
+    PureDistributedDataParallel,
+    ThreadWorld,
+)
+
+
+class MyModel(nn.Module):
+    def __init__(self) -> None:
+        super().__init__()
+        self.model = nn.Sequential(nn.Linear(3, 4), nn.Sigmoid())
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.model(x)
+
+
+class InjectedFailure(Exception):
+    pass
+
+
+class FailureInjector:
+    def __init__(self) -> None:
+        self._lock = threading.Lock()
+        self._failures = set()
+        self.count = 0
+
+    def fail_at(self, rank: int, step: int) -> "FailureInjector":
+        with self._lock:
+            self._failures.add((rank, step))
+            return self
+
+    def check(self, rank: int, step: int) -> None:
+        with self._lock:
+            key = (rank, step)
+            if key in self._failures:
+                self.count += 1
+                self._failures.remove(key)
+                raise InjectedFailure(f"injected failure {rank=} {step=}")
+
+
+class Runner:
+    def __init__(self, replica_id: int, lighthouse: InProcessLighthouse, world: ThreadWorld,
+                 injector: FailureInjector, train_loop: Callable, device: torch.device,
+                 init_state: Dict[str, torch.Tensor], use_async_quorum: bool = True,
+                 attempts: int = 3) -> None:
+        self.replica_id = replica_id
+        self.lighthouse = lighthouse
+        self.world = world
+        self.injector = injector
+        self.train_loop = train_loop
+        self.device = device
+        self.init_state = init_state
+        self.use_async_quorum = use_async_quorum
+        self.attempts = attempts
+
+    def make_manager(self, load_state_dict, state_dict) -> Manager:
+        self.client = self.lighthouse.client(f"replica_{self.replica_id}")
+        return Manager(
+            pg=ProcessGroupThreads(self.world),
+            load_state_dict=load_state_dict,
+            state_dict=state_dict,
+            min_replica_size=2,
+            use_async_quorum=self.use_async_quorum,
+            timeout=timedelta(seconds=20),
+            quorum_timeout=timedelta(seconds=30),
+            replica_id=str(self.replica_id),
+            checkpoint_transport=CheckpointServer(timeout=timedelta(seconds=20)),
+            quorum_client=self.client,
+        )
+
+    def run_replica(self):
+        for attempt in range(self.attempts):
+            manager: Optional[Manager] = None
+            try:
+                return self.train_loop(self)
+            except InjectedFailure as e:
+                print(f"replica {self.replica_id} attempt {attempt}: {e}", flush=True)
+                if attempt == self.attempts - 1:
+                    raise
+            finally:
+                self.client.leave()
+                if getattr(self, "manager", None) is not None:
+                    self.manager.shutdown(wait=False)
+        raise RuntimeError("ran out of attempts")
+
+
+def ddp_train_loop(runner: Runner):
+    torch.cuda.set_device(runner.device) if runner.device.type == "cuda" else None
+    m = MyModel().to(runner.device)
+    m.load_state_dict(runner.init_state if runner.replica_id == 0 else
+                      {k: torch.zeros_like(v) for k, v in runner.init_state.items()})
+    optimizer = optim.Adam(m.parameters())
+
+    def load_state_dict(sd):
+        m.load_state_dict(sd["model"])
+        optimizer.load_state_dict(sd["optim"])
+
+    def state_dict():
+        return {"model": m.state_dict(), "optim": optimizer.state_dict()}
+
+    manager = runner.manager = runner.make_manager(load_state_dict, state_dict)
+    # torch's Reducer waits for the hook's future on the autograd engine's per-device
+    # thread, which thread-replicas of one GPU share: there the Reducer-free wrapper is used
+    wrapper = PureDistributedDataParallel if runner.device.type == "cuda" else DistributedDataParallel
+    ddp = wrapper(manager, m)
+    wrapped = OptimizerWrapper(manager, optimizer)
+    criterion = nn.CrossEntropyLoss()
+    while True:
+        inputs = torch.rand(2, 3, device=runner.device)
+        labels = torch.randint(4, (2,), device=runner.device)
+        wrapped.zero_grad()
+        loss = criterion(ddp(inputs), labels)
+        loss.backward()
+        wrapped.step()
+        if manager.current_step() >= 4:
+            break
+        runner.injector.check(runner.replica_id, manager.current_step())
+    return {k: v.detach().cpu().clone() for k, v in m.state_dict().items()}, manager.current_step()
+
+
+def _sync_loop(runner: Runner, kind: str):
+    torch.cuda.set_device(runner.device) if runner.device.type == "cuda" else None
+    m = MyModel().to(runner.device)
+    m.load_state_dict(runner.init_state)
+    inner = optim.AdamW(m.parameters(), lr=4e-4, weight_decay=0.1, betas=(0.9, 0.95))
+    outer = optim.SGD(m.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    holder = {}
+
+    def load_state_dict(sd):
+        m.load_state_dict(sd["model"])
+        holder["sync"]._backup_parameters = sd["backup_params"]
+        inner.load_state_dict(sd["inner_optim"])
+        outer.load_state_dict(sd["outer_optim"])
+
+    def state_dict():
+        return {
+            "model": m.state_dict(),
+            "backup_params": copy.deepcopy(holder["sync"]._backup_parameters),
+            "inner_optim": inner.state_dict(),
+            "outer_optim": outer.state_dict(),
+        }
+
+    manager = runner.manager = runner.make_manager(load_state_dict, state_dict)
+    criterion = nn.CrossEntropyLoss()
+    history = {}
+    ctx = (DiLoCo(manager, m, inner, outer, sync_every=2) if kind == "diloco"
+           else LocalSGD(manager, m, inner, sync_every=2))
+    with ctx as sync:
+        holder["sync"] = sync
+        while True:
+            inputs = torch.rand(2, 3, device=runner.device)
+            labels = torch.randint(4, (2,), device=runner.device)
+            inner.zero_grad()
+            criterion(m(inputs), labels).backward()
+            inner.step()
+            snap = state_dict()
+            history[manager.current_step()] = {
+                "backup_params": {k: v.detach().cpu().clone() for k, v in snap["backup_params"].items()},
+                "outer_momentum": [st["momentum_buffer"].detach().cpu().clone()
+                                   for st in snap["outer_optim"]["state"].values()
+                                   if "momentum_buffer" in st],
+                "model": {k: v.detach().cpu().clone() for k, v in snap["model"].items()},
+            }
+            if manager.current_step() >= 4:
+                break
+            runner.injector.check(runner.replica_id, manager.current_step())
+    return history, manager.current_step()
+
+
+def diloco_train_loop(runner: Runner):
+    return _sync_loop(runner, "diloco")
+
+
+def local_sgd_train_loop(runner: Runner):
+    return _sync_loop(runner, "local_sgd")
+
+
+def run_cluster(train_loop: Callable, device: torch.device, injectors: List[FailureInjector],
+                use_async_quorum: bool = True):
+    lighthouse = InProcessLighthouse(min_replicas=2)
+    world = ThreadWorld()
+    torch.manual_seed(42)
+    init_state = {k: v.to(device) for k, v in MyModel().state_dict().items()}
+    runners = [Runner(i, lighthouse, world, inj, train_loop, device, init_state, use_async_quorum)
+               for i, inj in enumerate(injectors)]
+    results = [None] * len(runners)
+    with ThreadPoolExecutor(max_workers=len(runners)) as pool:
+        futures = {pool.submit(r.run_replica): i for i, r in enumerate(runners)}
+        for fut in as_completed(futures, timeout=120):
+            results[futures[fut]] = fut.result()
+    return results

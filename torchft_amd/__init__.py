@@ -9,6 +9,7 @@ declared in ``include/torchft_amd.h``; there is no CPU fallback.
 
 from .checkpointing import CheckpointServer, CheckpointTransport
 from .ddp import DistributedDataParallel, GradBucketAverager, PureDistributedDataParallel
+from .local_cluster import InProcessLighthouse, ProcessGroupThreads, ThreadWorld
 from .local_sgd import DiLoCo, LocalSGD
 from .manager import (
     Manager,
@@ -32,6 +33,7 @@ __all__ = (
     "DiLoCo",
     "DistributedDataParallel",
     "GradBucketAverager",
+    "InProcessLighthouse",
     "LocalSGD",
     "Manager",
     "ManagerClientAdapter",
@@ -40,9 +42,11 @@ __all__ = (
     "ProcessGroup",
     "ProcessGroupDummy",
     "ProcessGroupLocalReplicas",
+    "ProcessGroupThreads",
     "PureDistributedDataParallel",
     "QuorumClient",
     "QuorumResult",
     "StaticQuorum",
+    "ThreadWorld",
     "WorldSizeMode",
 )
