@@ -3,8 +3,8 @@
 // Every kernel here is HBM-bound elementwise work over a table of tensors.  The
 // table is cut into chunks (a power-of-two number of elements of one tensor) and
 // every chunk into slabs; one workgroup of 256 lanes (4 wavefronts of 64) owns
-// exactly one slab: one 128-bit access per lane and per stream, i.e. 4 KiB per
-// stream.  A workgroup finds its tensor with one scalar lookup
+// exactly one slab: one, two or four 128-bit accesses per lane and per stream,
+// i.e. 4-16 KiB per stream.  A workgroup finds its tensor with one scalar lookup
 // (chunk_tensor[blockIdx >> shift]) followed by one round of scalar loads of
 // that tensor's pointers.  Slabs are deliberately tiny and handed out by the
 // hardware dispatcher in order: the set of workgroups in flight then covers a
@@ -29,7 +29,6 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kMaxCols = TFT_MAX_REPLICAS + 3;
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 thread_local char g_err[512] = "";
