@@ -289,6 +289,25 @@ def bench_localsgd(args) -> Dict[str, object]:
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
     out["roofline"] = roofline(n_params * 4 * (n_rep + 2), kernel_ms,
                                "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>")
+    if not args.no_cpu_baseline:
+        from oracle import replica_sync as O
+
+        cpu_shapes = workloads.llama3_8b_shapes(args.cpu_layers, with_embeddings=False)
+        cw = workloads.make_diloco_workload(cpu_shapes, n_rep, dev)
+        backup = [t.cpu() for t in cw.backup]
+        reps = [[t.cpu() for t in rep] for rep in cw.replicas]
+        del cw
+        O.localsgd_perform_sync(reps, backup, [True] * n_rep, n_rep, True)
+        t0 = time.perf_counter()
+        for _ in range(args.cpu_steps):
+            O.localsgd_perform_sync(reps, backup, [True] * n_rep, n_rep, True)
+        dt = (time.perf_counter() - t0) / args.cpu_steps
+        n_cpu = sum(t.numel() for t in backup)
+        out["cpu_baseline"] = {
+            "value": n_cpu / dt, "unit": "params/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{args.cpu_layers} of 32 decoder layers (no embeddings), {args.cpu_steps} steps after "
+                      f"1 warm-up; {n_cpu} params, {dt * 1e3:.1f} ms/step; per-tensor torch CPU ops "
+                      f"(sum of replicas, divide, backup copy)"}
     return out
 
 
@@ -315,6 +334,25 @@ def bench_ddp_buckets(args) -> Dict[str, object]:
                      "n_buckets": len(averager.buckets), "n_elements": n_elems})
     out["roofline"] = roofline(n_elems * 2 * (3 + 1), kernel_ms,
                                "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets))
+    if not args.no_cpu_baseline:
+        from oracle import replica_sync as O
+
+        cpu_shapes = workloads.llama3_8b_shapes(args.cpu_layers, with_embeddings=False)
+        cg = [[t.cpu() for t in rep]
+              for rep in workloads.make_grad_replicas(cpu_shapes, 4, dev, torch.bfloat16)]
+        buckets = O.bucket_assignment([t.numel() for t in cg[0]], 2)
+        flags = [True, True, True, False]
+        O.ddp_bucket_average(cg, flags, 3, buckets)
+        t0 = time.perf_counter()
+        for _ in range(args.cpu_steps):
+            O.ddp_bucket_average(cg, flags, 3, buckets)
+        dt = (time.perf_counter() - t0) / args.cpu_steps
+        n_cpu = sum(t.numel() for t in cg[0])
+        out["cpu_baseline"] = {
+            "value": n_cpu / dt, "unit": "elements/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{args.cpu_layers} of 32 decoder layers (no embeddings), {len(buckets)} buckets, "
+                      f"{args.cpu_steps} steps after 1 warm-up; {n_cpu} elements, {dt * 1e3:.1f} ms/step; "
+                      f"torch CPU ops: flatten (cat), zero the spare, bf16 sum, divide, unflatten"}
     return out
 
 
@@ -371,6 +409,24 @@ def bench_checkpoint(args) -> Dict[str, object]:
                      "n_tensors": len(entries), "payload_bytes": payload})
     out["roofline"] = roofline(2 * payload, pack_ms, "mt_copy_kernel (pack)")
     out["unpack"] = roofline(2 * payload, unpack_ms, "mt_copy_kernel (unpack)")
+    if not args.no_cpu_baseline:
+        from oracle import replica_sync as O
+
+        del outs, srcs, table, staging
+        torch.cuda.empty_cache()
+        small = workloads.make_training_state(workloads.llama3_8b_shapes(1, with_embeddings=False), dev)
+        small_bytes = sum(e.nbytes for e in state_pack.plan_pack(small).entries)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        O.state_dict_round_trip(small)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {
+            "value": small_bytes / dt / 1e9, "unit": "GB/s (payload bytes through save + load)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"training state of 1 of 32 decoder layers on the GPU ({small_bytes} bytes), one "
+                      f"torch.save into memory + torch.load (the reference's send / receive seats), "
+                      f"{dt:.2f} s; includes its per-storage device-to-host copies"}
     out["pcie"] = {"d2h_GBs": total / d2h_s / 1e9, "h2d_GBs": total / h2d_s / 1e9,
                    "d2h_s": d2h_s, "h2d_s": h2d_s, "bytes": total,
                    "note": "staging buffer through two 1 GiB pinned bounce buffers; PCIe-bound, "
