@@ -427,11 +427,41 @@ def bench_checkpoint(args) -> Dict[str, object]:
             "sample": f"training state of 1 of 32 decoder layers on the GPU ({small_bytes} bytes), one "
                       f"torch.save into memory + torch.load (the reference's send / receive seats), "
                       f"{dt:.2f} s; includes its per-storage device-to-host copies"}
+    out["http_recovery"] = http_recovery(dev)
     out["pcie"] = {"d2h_GBs": total / d2h_s / 1e9, "h2d_GBs": total / h2d_s / 1e9,
                    "d2h_s": d2h_s, "h2d_s": h2d_s, "bytes": total,
                    "note": "staging buffer through two 1 GiB pinned bounce buffers; PCIe-bound, "
                            "reported separately from the HBM-bound kernels"}
     return out
+
+
+def http_recovery(dev: torch.device) -> Dict[str, object]:
+    """Live recovery end to end on a bounded slice: CheckpointServer.send_checkpoint on one
+    side, recv_checkpoint on the other (same process, loopback HTTP): device-side pack,
+    chunked pinned D2H, socket, chunked pinned H2D, views on the receiving GPU."""
+    from datetime import timedelta
+
+    from torchft_amd import CheckpointServer, state_pack, workloads
+
+    state = workloads.make_training_state(workloads.llama3_8b_shapes(3, with_embeddings=False), dev)
+    nbytes = sum(e.nbytes for e in state_pack.plan_pack(state).entries)
+    server = CheckpointServer(timeout=timedelta(seconds=120))
+    try:
+        server.send_checkpoint([1], 1, state, timedelta(seconds=120))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        got = server.recv_checkpoint(0, server.metadata(), 1, timedelta(seconds=120))
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        name = next(iter(state["user"]["model"]))
+        if not torch.equal(got["user"]["model"][name], state["user"]["model"][name]):
+            raise RuntimeError("recovered state differs")
+    finally:
+        server.shutdown()
+    return {"GBs": nbytes / dt / 1e9, "seconds": dt, "bytes": nbytes,
+            "note": "training state of 3 decoder layers served and fetched over loopback HTTP in one "
+                    "process (Python socket I/O bound); the reference's torch.save / torch.load seats "
+                    "are timed in cpu_baseline"}
 
 
 def main() -> int:
