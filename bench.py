@@ -55,6 +55,9 @@ def parse_args() -> argparse.Namespace:
                     help="run one plain multi-tensor copy of known size before the timed loop "
                          "(reference point for hardware-counter runs)")
     ap.add_argument("--variant", type=int, default=0, help="launch variant (tuning; 0 = default)")
+    ap.add_argument("--arena", action="store_true",
+                    help="carve all tensors of the DiLoCo workload out of one device allocation "
+                         "instead of allocating each separately (makes no measurable difference)")
     return ap.parse_args()
 
 
@@ -160,9 +163,32 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         shapes, n_rep = workloads.llama3_8b_shapes(), 2
     else:
         shapes, n_rep = workloads.gpt2_small_shapes(), 4
-    wl = workloads.make_diloco_workload(shapes, n_rep, dev)
-    params = [torch.empty_like(t) for t in wl.backup]
-    bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
+    if args.arena:
+        per_set = sum(-(-workloads.numel(sh) * 4 // 256) * 256 for _, sh in shapes)
+        arena = torch.empty((3 + n_rep) * per_set, dtype=torch.uint8, device=dev)
+        cursor = [0]
+
+        def carve(like):
+            out = []
+            for t in like:
+                n = t.numel() * 4
+                v = arena[cursor[0]:cursor[0] + n].view(torch.float32).view(t.shape)
+                v.copy_(t)
+                out.append(v)
+                cursor[0] += -(-n // 256) * 256
+            return out
+
+        backup = carve(workloads.normal_tensors(shapes, 0.02, workloads.SEED_BACKUP, dev))
+        replicas = [carve(workloads.drifted_replica(backup, 1e-3, workloads.SEED_REPLICA + r))
+                    for r in range(n_rep)]
+        wl = workloads.DilocoWorkload([n for n, _ in shapes], backup, replicas)
+        params = carve([torch.zeros(1, device=dev).expand(workloads.numel(sh)).view(sh) for _, sh in shapes])
+        bufs = carve(workloads.normal_tensors(shapes, 1e-3, 4000, dev))
+        torch.cuda.empty_cache()
+    else:
+        wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+        params = [torch.empty_like(t) for t in wl.backup]
+        bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
     sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
     table = TensorTable([params, wl.backup, bufs, *wl.replicas], what="bench")
     torch.cuda.synchronize()
@@ -208,7 +234,9 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         {"workload": f"DiLoCo outer step, fp32, {which}-shaped params ({len(shapes)} tensors, "
                      f"{n_params} params), {n_rep} simulated replicas, Nesterov SGD lr={LR} "
                      f"momentum={MOMENTUM}, one fused multi-tensor launch per step",
-         "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
+         "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
+         "allocation": ("every tensor is a contiguous view carved out of one device allocation"
+                        if args.arena else "one device allocation per tensor")})
     out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>")
     if reseeds[0]:
         out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]

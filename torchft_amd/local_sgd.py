@@ -136,6 +136,9 @@ class LocalSGD:
         assert sync_every >= 1, "sync_every must be greater than or equal to 1"
         self._backup_parameters: Dict[str, torch.Tensor] = {}
         self._host_backup: Optional[_PackedHostBackup] = None
+        self._hooks: List[RemovableHandle] = []
+        self._tables: Dict[str, TensorTable] = {}
+        self._flat: Dict[str, tuple] = {}
         named = list(self._model.named_parameters())
         if (
             backup_device is not None
@@ -147,6 +150,15 @@ class LocalSGD:
             self._host_backup = _PackedHostBackup(named, pin_memory)
             for (name, _), view in zip(named, self._host_backup.host_views):
                 self._backup_parameters[name] = view
+        elif (
+            named
+            and all(p.is_cuda and p.device == named[0][1].device for _, p in named)
+            and (backup_device is None or torch.device(backup_device) == named[0][1].device)
+        ):
+            # backup in HBM next to the parameters: views into one allocation per dtype
+            _, views = self._flat_like("backup", [p.data for _, p in named])
+            for (name, _), view in zip(named, views):
+                self._backup_parameters[name] = view
         else:
             for name, p in named:
                 device = backup_device if backup_device is not None else p.device
@@ -156,9 +168,6 @@ class LocalSGD:
                 self._backup_parameters[name] = t
         if named and any(p.is_cuda for _, p in named):
             _native.lib()  # GPU parameters need the kernels: fail now, loudly, if they are missing
-        self._hooks: List[RemovableHandle] = []
-        self._tables: Dict[str, TensorTable] = {}
-        self._flat: Dict[str, tuple] = {}
         # the first sync needs a valid backup
         self._save_parameters()
 
@@ -390,7 +399,8 @@ class DiLoCo(LocalSGD):
         not yet part of the optimizer state (see ``_attach_momentum``)."""
         live = [p for p in self._model.parameters()]
         if first:
-            return [torch.empty_like(live[i].data) for i in idx]
+            key = "momentum/" + ",".join(map(str, idx[:4])) + f"/{len(idx)}"
+            return self._flat_like(key, [live[i].data for i in idx])[1]
         return [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
 
     def _attach_momentum(self, idx: Sequence[int], bufs: Sequence[torch.Tensor]) -> None:
