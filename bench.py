@@ -55,6 +55,10 @@ def parse_args() -> argparse.Namespace:
                     help="run one plain multi-tensor copy of known size before the timed loop "
                          "(reference point for hardware-counter runs)")
     ap.add_argument("--variant", type=int, default=0, help="launch variant (tuning; 0 = default)")
+    ap.add_argument("--settle-seconds", type=float, default=8.0,
+                    help="idle this long before the first device allocation: device memory freed by a "
+                         "process that has just exited is handed out in a worse physical layout for a "
+                         "few seconds (2-5 %% lower bandwidth for the whole run); 0 disables")
     ap.add_argument("--arena", action="store_true",
                     help="carve all tensors of the DiLoCo workload out of one device allocation "
                          "instead of allocating each separately (makes no measurable difference)")
@@ -502,6 +506,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
+    if args.settle_seconds > 0:
+        time.sleep(args.settle_seconds)  # before anything is allocated on the device
     torch.cuda.set_device(0)
     from torchft_amd import ops
 
