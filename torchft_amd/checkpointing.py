@@ -97,7 +97,13 @@ class CheckpointServer(CheckpointTransport[T]):
     with the training thread's later work.
     """
 
-    def __init__(self, timeout: timedelta, chunk_bytes: int = state_pack.DEFAULT_CHUNK_BYTES) -> None:
+    def __init__(
+        self,
+        timeout: timedelta,
+        chunk_bytes: int = state_pack.DEFAULT_CHUNK_BYTES,
+        allow_pickle: bool = True,
+    ) -> None:
+        self._allow_pickle = allow_pickle
         self._checkpoint_lock = threading.Lock()
         self._disallowed = False
         self._step = -1
@@ -177,13 +183,14 @@ class CheckpointServer(CheckpointTransport[T]):
 
     # -- fetching ------------------------------------------------------------
     @classmethod
-    def load_from_address(cls, address: str, timeout: timedelta) -> T:
+    def load_from_address(cls, address: str, timeout: timedelta, allow_pickle: bool = True) -> T:
         """Fetches and unpacks the state dict served at ``address``; device tensors are
-        rebuilt on the current GPU."""
+        rebuilt on the current GPU.  Nothing is unpickled unless the sender had to embed a
+        leaf that JSON cannot express (``allow_pickle=False`` refuses such a state)."""
         logger.info("fetching checkpoint from %s", address)
         with urllib.request.urlopen(address, timeout=timeout.total_seconds()) as f:
             header, staging = state_pack.read_packed(f, None)
-        return state_pack.unpack(header, staging, copy=False)
+        return state_pack.unpack(header, staging, copy=False, allow_pickle=allow_pickle)
 
     def address(self) -> str:
         """``http://host:port/checkpoint/``; the step number is appended by the fetcher."""
@@ -226,4 +233,4 @@ class CheckpointServer(CheckpointTransport[T]):
         self.allow_checkpoint(step)
 
     def recv_checkpoint(self, src_rank: int, metadata: str, step: int, timeout: timedelta) -> T:
-        return self.load_from_address(f"{metadata}{step}", timeout)
+        return self.load_from_address(f"{metadata}{step}", timeout, self._allow_pickle)

@@ -13,18 +13,24 @@ Wire layout of a packed state::
 
     b"TFTPACK1" | u64 header_len | header | payload (header.total_bytes)
 
-``header`` is a pickle of ``{"skeleton", "entries", "total_bytes"}``: the state
-dict with every device tensor replaced by a ``TensorSlot(index)``; per slot the
-byte offset (256-byte aligned), dtype and shape.  Everything that is not a
-device tensor (ints, floats, strings, CPU tensors, param_groups, scheduler
-objects ...) travels inside the skeleton, as it does inside ``torch.save``'s
-pickle; like ``torch.load(weights_only=False)`` on the reference's receive path
-the header must therefore only be accepted from a trusted peer.
+``header`` is UTF-8 JSON ``{"skeleton", "entries", "total_bytes"}``: the state
+dict with every device tensor replaced by a slot number; per slot the byte
+offset (256-byte aligned), dtype and shape.  The skeleton carries dicts (any
+key type), lists, tuples, strings, numbers, booleans, None and CPU tensors
+(raw bytes, base64) as tagged JSON nodes, so an ordinary training state -
+model, optimizer state, param_groups, step counters - is rebuilt without
+unpickling anything.  A leaf JSON cannot express (an lr_scheduler object, say)
+is embedded as a pickle; the receiver only unpickles such leaves when called
+with ``allow_pickle=True``, which is the transport's default because the
+reference's receive path is ``torch.load(weights_only=False)``
+(torchft/checkpointing.py:201-203) and must keep working for such states.
 """
 
 from __future__ import annotations
 
+import base64
 import io
+import json
 import pickle
 import struct
 from collections import OrderedDict
@@ -116,10 +122,15 @@ class PackPlan:
     total_bytes: int
 
     def header(self) -> bytes:
-        return pickle.dumps(
-            {"skeleton": self.skeleton, "entries": self.entries, "total_bytes": self.total_bytes},
-            protocol=pickle.HIGHEST_PROTOCOL,
-        )
+        doc = {
+            "skeleton": _encode(self.skeleton),
+            "entries": [
+                [e.offset, e.nbytes, e.dtype, list(e.shape), e.requires_grad, e.is_parameter]
+                for e in self.entries
+            ],
+            "total_bytes": self.total_bytes,
+        }
+        return json.dumps(doc, separators=(",", ":")).encode("utf-8")
 
 
 def plan_pack(state_dict: Any) -> PackPlan:
@@ -183,25 +194,129 @@ def pack(
     return PackedState(plan, staging)
 
 
-def parse_header(header: bytes) -> Dict[str, Any]:
-    """Unpickles a header (trusted peers only, see the module docstring)."""
-    meta = pickle.loads(header)
-    if not isinstance(meta, dict) or set(meta) != {"skeleton", "entries", "total_bytes"}:
+_TAG = "__tft__"
+
+
+def _encode(obj: Any) -> Any:
+    """Skeleton -> JSON-able tree.  Plain JSON values stay as they are; everything else
+    becomes a ``{"__tft__": kind, ...}`` node."""
+    if obj is None or isinstance(obj, (bool, str)):
+        return obj
+    if isinstance(obj, int):
+        return obj if -(2 ** 53) < obj < 2 ** 53 else {_TAG: "int", "v": str(obj)}
+    if isinstance(obj, float):
+        return obj if obj == obj and obj not in (float("inf"), float("-inf")) else {
+            _TAG: "float", "v": repr(obj)}
+    if isinstance(obj, TensorSlot):
+        return {_TAG: "slot", "i": obj.index}
+    if isinstance(obj, torch.Tensor) and not isinstance(obj, torch.nn.Parameter) \
+            and obj.device.type == "cpu" and str(obj.dtype) in _DTYPES and not obj.is_sparse:
+        raw = obj.detach().contiguous().reshape(-1).view(torch.uint8).numpy().tobytes()
+        return {_TAG: "cpu_tensor", "dtype": str(obj.dtype), "shape": list(obj.shape),
+                "requires_grad": bool(obj.requires_grad),
+                "data": base64.b64encode(raw).decode("ascii")}
+    if type(obj) is dict and all(isinstance(k, str) and k != _TAG for k in obj):
+        return {k: _encode(v) for k, v in obj.items()}
+    if type(obj) in (dict, OrderedDict):  # keys of any hashable kind, order kept
+        return {_TAG: "odict" if type(obj) is OrderedDict else "dict",
+                "items": [[_encode(k), _encode(v)] for k, v in obj.items()]}
+    if type(obj) is list:
+        return [_encode(v) for v in obj]
+    if type(obj) is tuple:
+        return {_TAG: "tuple", "v": [_encode(v) for v in obj]}
+    blob = pickle.dumps(obj, protocol=pickle.HIGHEST_PROTOCOL)
+    return {_TAG: "pickle", "type": type(obj).__name__, "data": base64.b64encode(blob).decode("ascii")}
+
+
+def _decode(node: Any, allow_pickle: bool) -> Any:
+    if isinstance(node, list):
+        return [_decode(v, allow_pickle) for v in node]
+    if not isinstance(node, dict):
+        return node
+    kind = node.get(_TAG)
+    if kind is None:
+        return {k: _decode(v, allow_pickle) for k, v in node.items()}
+    if kind == "slot":
+        return TensorSlot(int(node["i"]))
+    if kind == "int":
+        return int(node["v"])
+    if kind == "float":
+        return float(node["v"])
+    if kind == "tuple":
+        return tuple(_decode(v, allow_pickle) for v in node["v"])
+    if kind in ("dict", "odict"):
+        out = OrderedDict() if kind == "odict" else {}
+        for k, v in node["items"]:
+            key = _decode(k, allow_pickle)
+            out[tuple(key) if isinstance(key, list) else key] = _decode(v, allow_pickle)
+        return out
+    if kind == "cpu_tensor":
+        dtype = _DTYPES[node["dtype"]]
+        raw = bytearray(base64.b64decode(node["data"]))
+        t = torch.frombuffer(raw, dtype=torch.uint8).clone() if raw else torch.empty(0, dtype=torch.uint8)
+        t = t.view(dtype).view(node["shape"])
+        return t.requires_grad_(True) if node.get("requires_grad") else t
+    if kind == "pickle":
+        if not allow_pickle:
+            raise ValueError(
+                f"the packed state holds a pickled {node.get('type', 'object')}; "
+                "pass allow_pickle=True to accept it (trusted peers only)"
+            )
+        return pickle.loads(base64.b64decode(node["data"]))
+    raise ValueError(f"unknown node kind {kind!r} in packed-state header")
+
+
+def header_total_bytes(header: bytes) -> int:
+    """Payload size announced by a header; decodes nothing else."""
+    try:
+        doc = json.loads(header.decode("utf-8"))
+        total = int(doc["total_bytes"])
+    except (UnicodeDecodeError, ValueError, KeyError, TypeError) as e:
+        raise ValueError(f"not a packed-state header: {e}") from None
+    if total < 0:
+        raise ValueError("not a packed-state header: negative payload size")
+    return total
+
+
+def parse_header(header: bytes, allow_pickle: bool = True) -> Dict[str, Any]:
+    """Decodes a header into ``{"skeleton", "entries", "total_bytes"}``.  Nothing is
+    unpickled unless the sender embedded a leaf JSON cannot express and
+    ``allow_pickle`` is true."""
+    try:
+        doc = json.loads(header.decode("utf-8"))
+    except (UnicodeDecodeError, ValueError) as e:
+        raise ValueError(f"not a packed-state header: {e}") from None
+    if not isinstance(doc, dict) or set(doc) != {"skeleton", "entries", "total_bytes"}:
         raise ValueError("not a packed-state header")
-    return meta
+    entries = [
+        TensorEntry(int(o), int(n), str(d), tuple(int(x) for x in sh), bool(rg), bool(ip))
+        for o, n, d, sh, rg, ip in doc["entries"]
+    ]
+    total = int(doc["total_bytes"])
+    for e in entries:
+        if e.dtype not in _DTYPES or e.offset < 0 or e.nbytes < 0 or e.offset + e.nbytes > total:
+            raise ValueError("packed-state header describes a tensor outside the payload")
+        numel = 1
+        for x in e.shape:
+            numel *= x
+        if numel * _DTYPES[e.dtype].itemsize != e.nbytes:
+            raise ValueError("packed-state header: shape and byte count disagree")
+    return {"skeleton": _decode(doc["skeleton"], allow_pickle), "entries": entries,
+            "total_bytes": total}
 
 
 def unpack(
     header: bytes,
     staging: Optional[torch.Tensor],
     copy: bool = True,
+    allow_pickle: bool = True,
 ) -> Any:
     """Rebuilds the state dict from ``header`` and the device-resident ``staging``.
 
     ``copy=True`` scatters into freshly allocated tensors with one kernel launch;
     ``copy=False`` returns views into ``staging`` (no traffic at all; the tensors
     then live as long as the staging buffer does)."""
-    meta = parse_header(header)
+    meta = parse_header(header, allow_pickle)
     entries: List[TensorEntry] = meta["entries"]
     if not entries:
         return _fill(meta["skeleton"], [])
@@ -295,7 +410,7 @@ def read_packed(
     header = src.read(hlen)
     if len(header) != hlen:
         raise EOFError("stream ended inside the header")
-    total = parse_header(header)["total_bytes"]
+    total = header_total_bytes(header)
     if total == 0:
         return header, None
     if device is None:
@@ -326,6 +441,6 @@ def dumps(state_dict: Any) -> bytes:
     return buf.getvalue()
 
 
-def loads(data: bytes, device: Optional[torch.device] = None) -> Any:
+def loads(data: bytes, device: Optional[torch.device] = None, allow_pickle: bool = True) -> Any:
     header, staging = read_packed(io.BytesIO(data), device)
-    return unpack(header, staging, copy=False)
+    return unpack(header, staging, copy=False, allow_pickle=allow_pickle)
