@@ -512,6 +512,14 @@ def main() -> int:
     from torchft_amd import ops
 
     ops.set_launch_variant(args.variant)
+    if args.calibration_copy and not args.workload.startswith("diloco_llama3_8b"):
+        # reference point for hardware-counter runs: a plain copy of exactly 8 GiB
+        src = torch.zeros(8 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        ops.mt_copy([dst], [src])
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     if args.workload == "diloco_llama3_8b":
         out = bench_diloco(args, "llama3_8b")
     elif args.workload == "diloco_gpt2_small":
