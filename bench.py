@@ -89,15 +89,20 @@ class Timed:
         return wall_ms, kernel_ms
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
-# each counter scaled by its reading for a plain copy of known size; the summary is kept
-# under profiles/).  Only the headline kernel has been measured.
-MEASURED_TRAFFIC_BYTES = {"mt_stream_kernel<F32, DilocoFusedOp<2>>": 224.810e9}
+# HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs per
+# workload, each counter scaled by its reading for a plain copy of known size; the
+# summaries are kept under profiles/).  Counters cannot be read from inside this script.
+MEASURED_TRAFFIC_BYTES = {
+    "diloco_llama3_8b": 224.810e9,        # 128.447 GB read + 96.363 GB written
+    "localsgd_llama3_8b": 128.483e9,      # 64.233 + 64.250
+    "ddp_buckets_llama3_8b": 64.263e9,    # 48.202 + 16.061, all 162 launches of a step
+    "diloco_gpt2_small": 3.608e9,         # 2.364 + 1.244 (partly served from cache)
+}
 
 
-def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1) -> Dict[str, object]:
+def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1,
+             traffic: object = None) -> Dict[str, object]:
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(kernel) if algo_bytes > 2e11 else None
     return {
         "bound": "hbm",
         "achieved": achieved,
@@ -241,7 +246,8 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
          "allocation": ("every tensor is a contiguous view carved out of one device allocation"
                         if args.arena else "one device allocation per tensor")})
-    out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>")
+    out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>",
+                               traffic=MEASURED_TRAFFIC_BYTES.get(f"diloco_{which}"))
     if reseeds[0]:
         out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]
         out["roofline"]["note"] = ("steps that re-seed the state include two extra copy launches in "
@@ -320,7 +326,8 @@ def bench_localsgd(args) -> Dict[str, object]:
                                  "params, 2 simulated replicas, one launch per step",
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
     out["roofline"] = roofline(n_params * 4 * (n_rep + 2), kernel_ms,
-                               "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>")
+                               "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>",
+                               traffic=MEASURED_TRAFFIC_BYTES["localsgd_llama3_8b"])
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
 
@@ -365,7 +372,8 @@ def bench_ddp_buckets(args) -> Dict[str, object]:
                                  "over per-parameter views (no flatten / unflatten passes)",
                      "n_buckets": len(averager.buckets), "n_elements": n_elems})
     out["roofline"] = roofline(n_elems * 2 * (3 + 1), kernel_ms,
-                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets))
+                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets),
+                               traffic=MEASURED_TRAFFIC_BYTES["ddp_buckets_llama3_8b"])
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
 
@@ -439,7 +447,7 @@ def bench_checkpoint(args) -> Dict[str, object]:
                                  f"exp_avg_sq + int64 steps, {len(entries)} device tensors, "
                                  f"{payload} bytes, one gather launch into a contiguous staging buffer",
                      "n_tensors": len(entries), "payload_bytes": payload})
-    out["roofline"] = roofline(2 * payload, pack_ms, "mt_copy_kernel (pack)")
+    out["roofline"] = roofline(2 * payload, pack_ms, "mt_copy_kernel (pack)", traffic=2.0 * payload)
     out["unpack"] = roofline(2 * payload, unpack_ms, "mt_copy_kernel (unpack)")
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
