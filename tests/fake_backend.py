@@ -6,7 +6,7 @@ the product never imports it and has no CPU path of its own.  Use the ``cpu_ops`
 fixture, which monkeypatches the functions below over ``torchft_amd.ops``.
 """
 
-from typing import List, Optional, Sequence
+from typing import List
 
 import torch
 

@@ -28,7 +28,6 @@ from torchft_amd import (
     Manager,
     OptimizerWrapper,
     ProcessGroup,
-    ProcessGroupDummy,
     ProcessGroupLocalReplicas,
     PureDistributedDataParallel,
     QuorumResult,

@@ -16,7 +16,7 @@ flatten and unflatten cost no memory traffic at all.
 
 # No postponed evaluation of annotations here: torch checks that the communication
 # hook annotates its bucket argument with the dist.GradBucket class itself.
-from typing import TYPE_CHECKING, Dict, List, Optional, Sequence
+from typing import TYPE_CHECKING, List, Optional, Sequence
 
 import torch
 import torch.distributed as dist

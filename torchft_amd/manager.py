@@ -29,7 +29,6 @@ from __future__ import annotations
 
 import concurrent.futures
 import logging
-import threading
 from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass, field
 from datetime import timedelta
@@ -461,10 +460,7 @@ class Manager(Generic[T]):
             return _done_future(tensors)
         self.wait_quorum()
         try:
-            per_tensor = [self._pg.ordered(t, self.is_participating()) for t in tensors]
-            mask = per_tensor[0][1] if per_tensor else 0
-            n_rep = len(per_tensor[0][0]) if per_tensor else 0
-            replicas = [[pt[0][r] for pt in per_tensor] for r in range(n_rep)]
+            replicas, mask = self.replica_columns(tensors)
             outs = [tensors] + ([list(also_write)] if also_write is not None else [])
             cols = [*outs, *replicas]
             key = "allreduce_tensors/%d" % len(outs)

@@ -9,7 +9,7 @@ copies (a whole small workload, or slices of a full-size one) to the other.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Sequence, Tuple
 
 import torch
 
