@@ -12,7 +12,8 @@
  *   - return 0 on success, a negative tft_status on error; tft_last_error()
  *     returns a thread-local message for the last failing call on this thread;
  *   - the library never allocates device memory, never synchronises and keeps
- *     no mutable global state: each call validates its arguments on the host
+ *     no mutable global state (the error string and the benchmark-only launch
+ *     variant are thread-local): each call validates its arguments on the host
  *     and enqueues exactly one kernel on the caller's hipStream_t (passed as
  *     void*; NULL is the legacy default stream);
  *   - re-entrant: may be called concurrently from the training thread, the
@@ -165,14 +166,15 @@ int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, v
  * (torchft/local_sgd.py:121-131), bucket flatten/unflatten (torch Reducer under
  * torchft/ddp.py:52-63) and checkpoint pack/unpack into one staging buffer
  * (the torch.save / torch.load seats at torchft/checkpointing.py:164,203).
- * dst and src of one tensor must not overlap.
+ * dst and src of one tensor must not overlap.  chunk_elems (bytes here) must be
+ * a power of two >= 16384.
  */
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream);
 
 /* Benchmark hook: selects a launch variant for later calls FROM THIS THREAD
- * (thread-local; 0 restores the tuned default).  bits 0-3: 128-bit accesses per
- * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; 0 = each kernel's tuned default);
- * bit 4: plain instead of non-temporal accesses. */
+ * (thread-local; 0 restores the tuned defaults).  bits 0-3: 128-bit accesses per
+ * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; 0 = each
+ * kernel's tuned default); bit 4: plain instead of non-temporal accesses. */
 void tft_set_launch_variant(uint32_t variant);
 
 #ifdef __cplusplus
