@@ -109,3 +109,17 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"columns" in lib.tft_last_error()
     # an empty table is a successful no-op
     assert lib.tft_mt_diloco_outer_f32(ctypes.byref(table), 2, 3, 2, ctypes.byref(sgd), None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No fallback: without the built library every entry into the native layer raises."""
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", tmp_path / "libtorchft_amd.so")
+    assert not _native.is_available()
+    with pytest.raises(_native.NativeLibraryError, match="is not built"):
+        _native.lib()
+    with pytest.raises(_native.NativeLibraryError):
+        multi_tensor.plan_chunks([10], 8192)
+    (tmp_path / "libtorchft_amd.so").write_bytes(b"not an ELF file")
+    with pytest.raises(_native.NativeLibraryError, match="cannot load"):
+        _native.lib()
