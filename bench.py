@@ -38,7 +38,8 @@ HBM_PEAK_GBS = 8000.0
 LR, MOMENTUM = 0.7, 0.9
 HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo"
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
-             "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api"]
+             "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
+             "diloco_two_phase_llama3_8b"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -307,6 +308,53 @@ def bench_diloco_api(args) -> Dict[str, object]:
     return out
 
 
+def bench_diloco_two_phase(args) -> Dict[str, object]:
+    """The two-phase form used when the commit decision must come between reduction and
+    update: phase 1 (pseudo-gradient average + restore, in place on replica 0) and phase 2
+    (outer SGD + backup refresh), each one launch, timed separately."""
+    from torchft_amd import ops, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes, n_rep = workloads.llama3_8b_shapes(), 2
+    wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+    params = wl.replicas[0]  # live parameters are replica 0
+    bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
+    grads = [torch.empty_like(t) for t in wl.backup]
+    sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
+    t1 = ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, True)
+    t2 = ops.mt_outer_sgd(params, wl.backup, bufs, grads, sgd, False)
+    pristine = [t.clone() for t in wl.backup]  # phase 2 moves the backup: put it back per step
+    torch.cuda.synchronize()
+    n_params = wl.n_params
+    e = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for i in range(args.warmup + args.steps):
+        k = i - args.warmup
+        ops.mt_copy(wl.backup, pristine)
+        ops.mt_copy(params, wl.replicas[1])  # some drift to average
+        if k >= 0:
+            e[k][0].record()
+        ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, True, table=t1)
+        if k >= 0:
+            e[k][1].record()
+        ops.mt_outer_sgd(params, wl.backup, bufs, grads, sgd, False, table=t2)
+        if k >= 0:
+            e[k][2].record()
+    torch.cuda.synchronize()
+    p1 = sum(a[0].elapsed_time(a[1]) for a in e) / args.steps
+    p2 = sum(a[1].elapsed_time(a[2]) for a in e) / args.steps
+    out = base_line(args, "two-phase DiLoCo sync params/sec, Llama-3-8B", n_params / ((p1 + p2) * 1e-3),
+                    "params/s", p1 + p2, "f32",
+                    {"workload": "DiLoCo sync in two launches (pseudo-gradient average + restore, then outer "
+                                 "SGD + backup refresh), Llama-3-8B fp32, 2 replicas, in place on replica 0; "
+                                 "ms_per_step is the sum of the two kernels (the state reset between steps "
+                                 "is not counted)",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
+    # phase 1: read x0, x1, b; write g, p.  phase 2: read g, b, buf; write p, b, buf.
+    out["roofline"] = roofline(n_params * 20, p1, "mt_stream_kernel<F32, PseudogradOp<2>>")
+    out["phase2"] = roofline(n_params * 24, p2, "mt_stream_kernel<F32, OuterSgdOp>")
+    return out
+
+
 def bench_localsgd(args) -> Dict[str, object]:
     from torchft_amd import ops, workloads
 
@@ -538,6 +586,8 @@ def main() -> int:
         out = bench_checkpoint(args)
     elif args.workload == "diloco_llama3_8b_api":
         out = bench_diloco_api(args)
+    elif args.workload == "diloco_two_phase_llama3_8b":
+        out = bench_diloco_two_phase(args)
     else:
         out = bench_localsgd(args)
     print(json.dumps(out), flush=True)
