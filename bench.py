@@ -55,11 +55,14 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one plain multi-tensor copy of known size before the timed loop "
                          "(reference point for hardware-counter runs)")
-    ap.add_argument("--variant", type=int, default=0, help="launch variant (tuning; 0 = default)")
     ap.add_argument("--settle-seconds", type=float, default=8.0,
                     help="idle this long before the first device allocation: device memory freed by a "
                          "process that has just exited is handed out in a worse physical layout for a "
                          "few seconds (2-5 %% lower bandwidth for the whole run); 0 disables")
+    ap.add_argument("--layout", default="",
+                    help="comma list for the DiLoCo workloads: alias_p (the live parameters are replica 0, "
+                         "updated in place), flat_backup / flat_momentum (backup / momentum tensors are "
+                         "views of one flat allocation, back to back without padding)")
     ap.add_argument("--arena", action="store_true",
                     help="carve all tensors of the DiLoCo workload out of one device allocation "
                          "instead of allocating each separately (makes no measurable difference)")
@@ -91,19 +94,28 @@ class Timed:
 
 
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs per
-# workload, each counter scaled by its reading for a plain copy of known size; the
-# summaries are kept under profiles/).  Counters cannot be read from inside this script.
-MEASURED_TRAFFIC_BYTES = {
-    "diloco_llama3_8b": 224.810e9,        # 128.447 GB read + 96.363 GB written
-    "localsgd_llama3_8b": 128.483e9,      # 64.233 + 64.250
-    "ddp_buckets_llama3_8b": 64.263e9,    # 48.202 + 16.061, all 162 launches of a step
-    "diloco_gpt2_small": 3.608e9,         # 2.364 + 1.244 (partly served from cache)
-}
+# workload, each counter scaled by its reading for a plain copy of known size).  Counters
+# cannot be read from inside this script: the figures, the scale factors and the commands
+# that produced them are kept in one tracked data file, which this script quotes.
+TRAFFIC_FILE = os.path.join(REPO_ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(workload: str) -> Tuple[object, object]:
+    """(HBM bytes per step from the hardware counters, where that figure comes from)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f)["workloads"][workload]
+        return float(entry["read_bytes"]) + float(entry["write_bytes"]), "profiles/hbm_traffic.json"
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1,
-             traffic: object = None) -> Dict[str, object]:
+             traffic: object = None, workload: str = "") -> Dict[str, object]:
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    source = None
+    if workload:
+        traffic, source = measured_traffic(workload)
     return {
         "bound": "hbm",
         "achieved": achieved,
@@ -111,6 +123,7 @@ def roofline(algo_bytes: float, kernel_ms: float, kernel: str, launches: int = 1
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic,
+        "traffic_source": source,
         "kernel": kernel,
         "kernel_ms_per_step": kernel_ms,
         "launches_per_step": launches,
@@ -199,6 +212,24 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         wl = workloads.make_diloco_workload(shapes, n_rep, dev)
         params = [torch.empty_like(t) for t in wl.backup]
         bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
+    layout = [x for x in args.layout.split(",") if x]
+    for item in layout:
+        if item == "alias_p":
+            params = wl.replicas[0]
+        elif item in ("flat_backup", "flat_momentum"):
+            src = wl.backup if item == "flat_backup" else bufs
+            flat = torch.empty(sum(t.numel() for t in src), dtype=torch.float32, device=dev)
+            views = ops.flat_views(flat, src)
+            ops.mt_copy(views, src)
+            torch.cuda.synchronize()
+            if item == "flat_backup":
+                wl.backup = views
+            else:
+                bufs = views
+            del src
+            torch.cuda.empty_cache()
+        else:
+            raise SystemExit(f"unknown --layout item {item!r}")
     sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
     table = TensorTable([params, wl.backup, bufs, *wl.replicas], what="bench")
     torch.cuda.synchronize()
@@ -246,9 +277,10 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
                      f"momentum={MOMENTUM}, one fused multi-tensor launch per step",
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
          "allocation": ("every tensor is a contiguous view carved out of one device allocation"
-                        if args.arena else "one device allocation per tensor")})
+                        if args.arena else "one device allocation per tensor"),
+         "layout": layout})
     out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>",
-                               traffic=MEASURED_TRAFFIC_BYTES.get(f"diloco_{which}"))
+                               workload=f"diloco_{which}")
     if reseeds[0]:
         out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]
         out["roofline"]["note"] = ("steps that re-seed the state include two extra copy launches in "
@@ -284,7 +316,7 @@ def bench_diloco_api(args) -> Dict[str, object]:
     peer = workloads.drifted_replica([p.data for p in model.parameters()], 1e-3, 1001)
     index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
     pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
                       quorum_client=StaticQuorum(0, 2))
     inner = torch.optim.SGD(model.parameters(), lr=0.1)
     outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
@@ -375,7 +407,7 @@ def bench_localsgd(args) -> Dict[str, object]:
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
     out["roofline"] = roofline(n_params * 4 * (n_rep + 2), kernel_ms,
                                "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>",
-                               traffic=MEASURED_TRAFFIC_BYTES["localsgd_llama3_8b"])
+                               workload="localsgd_llama3_8b")
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
 
@@ -421,7 +453,7 @@ def bench_ddp_buckets(args) -> Dict[str, object]:
                      "n_buckets": len(averager.buckets), "n_elements": n_elems})
     out["roofline"] = roofline(n_elems * 2 * (3 + 1), kernel_ms,
                                "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets),
-                               traffic=MEASURED_TRAFFIC_BYTES["ddp_buckets_llama3_8b"])
+                               workload="ddp_buckets_llama3_8b")
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
 
@@ -567,7 +599,6 @@ def main() -> int:
     torch.cuda.set_device(0)
     from torchft_amd import ops
 
-    ops.set_launch_variant(args.variant)
     if args.calibration_copy and not args.workload.startswith("diloco_llama3_8b"):
         # reference point for hardware-counter runs: a plain copy of exactly 8 GiB
         src = torch.zeros(8 << 30, dtype=torch.uint8, device="cuda")

@@ -12,10 +12,9 @@
  *   - return 0 on success, a negative tft_status on error; tft_last_error()
  *     returns a thread-local message for the last failing call on this thread;
  *   - the library never allocates device memory, never synchronises and keeps
- *     no mutable global state (the error string and the benchmark-only launch
- *     variant are thread-local): each call validates its arguments on the host
- *     and enqueues exactly one kernel on the caller's hipStream_t (passed as
- *     void*; NULL is the legacy default stream);
+ *     no mutable global state (the error string is thread-local): each call
+ *     validates its arguments on the host and enqueues exactly one kernel on the
+ *     caller's hipStream_t (passed as void*; NULL is the legacy default stream);
  *   - re-entrant: may be called concurrently from the training thread, the
  *     autograd thread (DDP comm hook) and the checkpoint thread.
  *
@@ -32,8 +31,11 @@
  *   it further into slabs of one 128-bit access per lane, one workgroup each.
  *   tft_mt_plan() computes both arrays on the host.  Tensors must be
  *   contiguous; columns of one tensor may alias each other only where a
- *   function says so.  Any alignment is accepted: a tensor whose columns are
- *   all 16-byte aligned takes the 128-bit path, others a scalar path.
+ *   function says so.  Any alignment is accepted: a tensor whose columns share
+ *   one misalignment (all 16-byte aligned, or all the same distance past a
+ *   16-byte boundary, as views into flat buffers are) runs with 128-bit accesses
+ *   after a scalar head of a few elements; columns misaligned differently from
+ *   each other take a scalar path.
  *
  * Arithmetic (fp32 unless noted; this is what "parity" means for this library)
  *   - the N replica contributions are added sequentially in replica order
@@ -54,7 +56,7 @@
 extern "C" {
 #endif
 
-#define TFT_ABI_VERSION 3
+#define TFT_ABI_VERSION 4
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
 #define TFT_MIN_CHUNK_ELEMS 8192u
 
@@ -133,17 +135,19 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
 /*
  * DiLoCo outer step, fully fused (torchft/local_sgd.py:205-225 with the commit
  * decision already known to be true).  Columns: [p, b, buf, replica_0 ..].
- * Per element:
+ * Per element, in fp32 (bf16 / fp16 storage is widened on load and rounded to
+ * nearest-even once on store; the reference runs the same torch ops in the
+ * tensors' own dtype, torchft/local_sgd.py:212-215 is dtype-generic):
  *   g    = (sum_r (replica_r - b)) / num_participants      (subtract, then sum)
  *   d    = weight_decay ? fma(b, weight_decay, g) : g
  *   buf' = first_step ? d : fma(d, 1 - dampening, momentum * buf)
  *   e    = nesterov ? fma(buf', momentum, d) : buf'    (momentum == 0: e = d, buf untouched)
  *   p = b = fma(e, -lr, b)
- * `p` may alias a replica column.  fp32 only.
+ * `p` may alias a replica column.
  */
-int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
-                            uint32_t participate_mask, uint32_t num_participants,
-                            const tft_sgd_params* sgd, void* stream);
+int tft_mt_diloco_outer(const tft_mt_table* table, uint32_t n_replicas, uint32_t participate_mask,
+                        uint32_t num_participants, int dtype, const tft_sgd_params* sgd,
+                        void* stream);
 
 /*
  * Two-phase form for callers that must consult should_commit() between the
@@ -154,11 +158,12 @@ int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
  *   `p` may alias a replica column; it is written after all reads.
  * Phase 2, columns [p, b, buf, g]: the SGD update above with g read from
  *   memory and the parameter value taken from b (p was restored to b).
+ * With bf16 / fp16 storage g is rounded once when phase 1 stores it.
  */
-int tft_mt_pseudograd_avg_f32(const tft_mt_table* table, uint32_t n_replicas,
-                              uint32_t participate_mask, uint32_t num_participants,
-                              int restore_p, void* stream);
-int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, void* stream);
+int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
+                          uint32_t participate_mask, uint32_t num_participants, int dtype,
+                          int restore_p, void* stream);
+int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd, void* stream);
 
 /*
  * Byte-exact multi-tensor gather/scatter.  Columns: [dst, src]; numel counts
@@ -170,12 +175,6 @@ int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, v
  * a power of two >= 16384.
  */
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream);
-
-/* Benchmark hook: selects a launch variant for later calls FROM THIS THREAD
- * (thread-local; 0 restores the tuned defaults).  bits 0-3: 128-bit accesses per
- * lane and stream, i.e. slab size in units of 4 KiB (1, 2 or 4; 0 = each
- * kernel's tuned default); bit 4: plain instead of non-temporal accesses. */
-void tft_set_launch_variant(uint32_t variant);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,11 @@ How each function is pinned (tests/test_oracle.py):
   diloco_perform_sync    composition check against torch.optim.SGD fed with a
                          float64-checked pseudo-gradient; fixed point; N=1
                          special case; cross-replica identity
-                         (torchft/manager_integ_test.py:553-562)
+                         (torchft/manager_integ_test.py:553-562); the
+                         fp32-arithmetic variant for bf16 / fp16 storage against
+                         a float64 evaluation (within one rounding of the storage
+                         dtype) and against the dtype-native form (the stated
+                         tolerance rtol 1e-2)
   localsgd_perform_sync  closed form mean; commit / no-commit invariants
                          (torchft/local_sgd_test.py:65-67, 98-101)
   bucket_assignment      torch's dist._compute_bucket_assignment_by_size and a
@@ -130,6 +134,8 @@ def diloco_perform_sync(
     dampening: float = 0.0,
     weight_decay: float = 0.0,
     nesterov: bool = False,
+    accumulate_dtype: Optional[torch.dtype] = None,
+    grads_through_storage: bool = False,
 ) -> Dict[str, List[Optional[torch.Tensor]]]:
     """``DiLoCo._perform_sync`` (torchft/local_sgd.py:205-225) for one replica group.
 
@@ -137,6 +143,15 @@ def diloco_perform_sync(
     (torchft/manager_integ_test.py:553-562) one result set is returned:
     ``{"params", "backup", "momentum", "grads"}``; ``grads`` is the averaged
     pseudo-gradient the reference stores in ``p.grad`` before ``zero_grad``.
+
+    ``accumulate_dtype=None`` is the reference itself: every torch op runs in the
+    tensors' own dtype (for bf16 parameters each subtraction, sum, division and
+    optimizer op rounds to bf16).  ``accumulate_dtype=torch.float32`` is the
+    fp32-arithmetic variant the kernels implement for 16-bit storage: the same
+    ops in the same order on values widened to fp32, each output rounded to the
+    storage dtype once.  ``grads_through_storage`` additionally rounds the
+    averaged pseudo-gradient to the storage dtype before the optimizer reads it
+    (the two-launch form, where it passes through memory between the launches).
     """
     n_tensors = len(backup)
     params: List[torch.Tensor] = []
@@ -144,21 +159,25 @@ def diloco_perform_sync(
     new_bufs: List[Optional[torch.Tensor]] = []
     grads: List[torch.Tensor] = []
     for t in range(n_tensors):
-        b = backup[t]
+        store = backup[t].dtype
+        work = accumulate_dtype or store
+        b = backup[t].detach().to(work)
         # local_sgd.py:212-215, on every replica
-        pseudo = [rp[t].detach() - b for rp in replica_params]
+        pseudo = [rp[t].detach().to(work) - b for rp in replica_params]
         # local_sgd.py:227-239 -> manager.py:267-287
         g = manager_allreduce_(pseudo, participating, num_participants)
-        p = b.detach().clone()  # local_sgd.py:219 (_restore_parameters)
-        buf = None if momentum_bufs is None or momentum_bufs[t] is None else momentum_bufs[t].clone()
-        nb = b.detach().clone()
+        if grads_through_storage:
+            g = g.to(store).to(work)
+        p = b.clone()  # local_sgd.py:219 (_restore_parameters)
+        buf = None if momentum_bufs is None or momentum_bufs[t] is None else momentum_bufs[t].to(work, copy=True)
+        nb = b.clone()
         if commit:  # local_sgd.py:221-224
             buf = sgd_step_(p, g, buf, lr, momentum, dampening, weight_decay, nesterov)
             nb = p.clone()
-        params.append(p)
-        new_backup.append(nb)
-        new_bufs.append(buf)
-        grads.append(g)
+        params.append(p.to(store))
+        new_backup.append(nb.to(store))
+        new_bufs.append(None if buf is None else buf.to(store))
+        grads.append(g.to(store))
     return {"params": params, "backup": new_backup, "momentum": new_bufs, "grads": grads}
 
 

@@ -42,3 +42,23 @@ def cpu_ops(monkeypatch):
     fake_backend.calls.clear()
     return fake_backend
 
+
+
+@pytest.fixture
+def launch_variant(monkeypatch):
+    """Routes the kernel wrappers through the tuning build of the library (same source,
+    compiled with -DTFT_TUNING, which exports the launch-shape override) and returns the
+    setter: bits 0-3 unroll (1, 2, 4), bit 4 plain accesses, bits 8-11 per-XCD run log2 + 1,
+    bits 12-15 LDS cap / 8 KiB + 1; 0 restores the built-in choice.  The override is
+    thread-local and is cleared when the test ends."""
+    import ctypes
+
+    from torchft_amd import _build, _native
+
+    handle = _native.load(_build.TUNING_LIB_PATH,
+                          {"tft_set_launch_variant": (None, [ctypes.c_uint32])})
+    monkeypatch.setattr(_native, "_lib", handle)
+    try:
+        yield handle.tft_set_launch_variant
+    finally:
+        handle.tft_set_launch_variant(0)

@@ -38,6 +38,10 @@ def reduce_avg_(out, replicas, participate_mask=None, num_participants=None):
     return out
 
 
+def check_tensor(t, what):
+    pass  # the stand-in computes on CPU tensors of any dtype
+
+
 def reduce_avg_table(outs, replicas):
     return FakeTable()
 
@@ -54,6 +58,13 @@ def mt_reduce_avg(outs, replicas, participate_mask=None, num_participants=None, 
     return FakeTable()
 
 
+def _pseudograd_f32(t, backups, replicas, mask, nump):
+    n = len(replicas)
+    b = backups[t].float()
+    pseudo = [rep[t].float() - b for rep in replicas]
+    return O.manager_allreduce_(pseudo, _flags(mask, n), nump)
+
+
 def mt_pseudograd_avg(grads, params, backups, replicas, restore_params, participate_mask=None,
                       num_participants=None, table=None):
     calls.append("mt_pseudograd_avg")
@@ -61,33 +72,43 @@ def mt_pseudograd_avg(grads, params, backups, replicas, restore_params, particip
     mask = real_ops.full_mask(n) if participate_mask is None else participate_mask
     nump = n if num_participants is None else num_participants
     for t in range(len(grads)):
-        pseudo = [rep[t] - backups[t] for rep in replicas]
-        grads[t].copy_(O.manager_allreduce_(pseudo, _flags(mask, n), nump))
+        grads[t].copy_(_pseudograd_f32(t, backups, replicas, mask, nump))  # one rounding on store
         if restore_params:
             params[t].copy_(backups[t])
     return FakeTable()
 
 
+def _sgd_from_backup(t, params, backups, bufs, g32, sgd, first_step):
+    p = backups[t].float()
+    buf = None if (first_step or bufs is None) else bufs[t].float()
+    buf = O.sgd_step_(p, g32, buf, sgd.lr, sgd.momentum, sgd.dampening, sgd.weight_decay,
+                      sgd.nesterov)
+    if bufs is not None and buf is not None:
+        bufs[t].copy_(buf)
+    params[t].copy_(p)
+    backups[t].copy_(p)
+
+
 def mt_outer_sgd(params, backups, bufs, grads, sgd, first_step, table=None):
     calls.append("mt_outer_sgd")
     for t in range(len(params)):
-        p = backups[t].clone()
-        buf = None if (first_step or bufs is None) else bufs[t]
-        buf = O.sgd_step_(p, grads[t], buf, sgd.lr, sgd.momentum, sgd.dampening,
-                          sgd.weight_decay, sgd.nesterov)
-        if bufs is not None and buf is not None:
-            bufs[t].copy_(buf)
-        params[t].copy_(p)
-        backups[t].copy_(p)
+        _sgd_from_backup(t, params, backups, bufs, grads[t].float(), sgd, first_step)
+    return FakeTable()
+
+
+def diloco_outer_table(params, backups, bufs, replicas, table=None):
     return FakeTable()
 
 
 def mt_diloco_outer(params, backups, bufs, replicas, sgd, first_step, participate_mask=None,
                     num_participants=None, table=None):
     calls.append("mt_diloco_outer")
-    grads = [torch.empty_like(b) for b in backups]
-    mt_pseudograd_avg(grads, params, backups, replicas, False, participate_mask, num_participants)
-    mt_outer_sgd(params, backups, bufs, grads, sgd, first_step)
+    n = len(replicas)
+    mask = real_ops.full_mask(n) if participate_mask is None else participate_mask
+    nump = n if num_participants is None else num_participants
+    for t in range(len(params)):
+        g32 = _pseudograd_f32(t, backups, replicas, mask, nump)  # stays in fp32 registers
+        _sgd_from_backup(t, params, backups, bufs, g32, sgd, first_step)
     return FakeTable()
 
 
@@ -98,5 +119,5 @@ def mt_copy(dsts, srcs, table=None):
     return FakeTable()
 
 
-PATCHED = ["reduce_avg_", "reduce_avg_table", "mt_reduce_avg", "mt_pseudograd_avg", "mt_outer_sgd",
-           "mt_diloco_outer", "mt_copy"]
+PATCHED = ["check_tensor", "reduce_avg_", "reduce_avg_table", "mt_reduce_avg", "mt_pseudograd_avg", "mt_outer_sgd",
+           "mt_diloco_outer", "diloco_outer_table", "mt_copy"]

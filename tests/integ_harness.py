@@ -165,8 +165,35 @@ def _sync_loop(runner: Runner, kind: str):
     history = {}
     ctx = (DiLoCo(manager, m, inner, outer, sync_every=2) if kind == "diloco"
            else LocalSGD(manager, m, inner, sync_every=2))
+    records = []
     with ctx as sync:
         holder["sync"] = sync
+        perform = sync._perform_sync
+
+        def cpu(ts):
+            return [t.detach().cpu().clone() for t in ts]
+
+        def momentum():
+            bufs = [outer.state.get(p, {}).get("momentum_buffer") for p in m.parameters()]
+            return None if any(b is None for b in bufs) else cpu(bufs)
+
+        def recording_perform_sync():
+            # once the quorum (and a synchronous heal) is done these are the sync's inputs
+            manager.wait_quorum()
+            names = [n for n, _ in m.named_parameters()]
+            rec = dict(step=manager.current_step(), params=cpu(m.parameters()),
+                       backup=cpu(sync._backup_parameters[n] for n in names), momentum=momentum())
+            perform()
+            rec.update(rank=manager._pg._rank, world=manager._pg._size,
+                       participating=manager.is_participating(),
+                       num_participants=manager.num_participants(),
+                       committed=manager.current_step() == rec["step"] + 1,
+                       post_params=cpu(m.parameters()),
+                       post_backup=cpu(sync._backup_parameters[n] for n in names),
+                       post_momentum=momentum())
+            records.append(rec)
+
+        sync._perform_sync = recording_perform_sync
         while True:
             inputs = torch.rand(2, 3, device=runner.device)
             labels = torch.randint(4, (2,), device=runner.device)
@@ -184,7 +211,7 @@ def _sync_loop(runner: Runner, kind: str):
             if manager.current_step() >= 4:
                 break
             runner.injector.check(runner.replica_id, manager.current_step())
-    return history, manager.current_step()
+    return history, manager.current_step(), records
 
 
 def diloco_train_loop(runner: Runner):

@@ -39,6 +39,16 @@ def test_library_exports_every_declared_symbol():
     assert {n for n in exported if n.startswith("tft_")} == set(declared_functions())
 
 
+def test_tuning_build_adds_only_the_launch_shape_override():
+    from torchft_amd import _build
+
+    out = subprocess.run(["nm", "-D", "--defined-only", str(_build.TUNING_LIB_PATH)],
+                         check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    assert {n for n in exported if n.startswith("tft_")} == \
+        set(declared_functions()) | {"tft_set_launch_variant"}
+
+
 def test_abi_version_and_constants():
     lib = _native.lib()
     text = open(HEADER).read()
@@ -102,13 +112,14 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.tft_reduce_avg(None, None, 1, 1, 1, 0, 0, None) == 0  # nothing to do
     table = _native.MtTable(None, None, None, None, 0, 5, 65536, 0)
     sgd = _native.SgdParams(0.7, 0.0, 0.0, 0.0, 1, 0)  # nesterov without momentum
-    assert lib.tft_mt_diloco_outer_f32(ctypes.byref(table), 2, 3, 2, ctypes.byref(sgd), None) == -1
+    assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, 0, ctypes.byref(sgd), None) == -1
     assert b"nesterov" in lib.tft_last_error()
     sgd = _native.SgdParams(0.7, 0.9, 0.0, 0.0, 1, 0)
-    assert lib.tft_mt_diloco_outer_f32(ctypes.byref(table), 3, 7, 3, ctypes.byref(sgd), None) == -1
+    assert lib.tft_mt_diloco_outer(ctypes.byref(table), 3, 7, 3, 0, ctypes.byref(sgd), None) == -1
     assert b"columns" in lib.tft_last_error()
+    assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, 9, ctypes.byref(sgd), None) == -2  # dtype
     # an empty table is a successful no-op
-    assert lib.tft_mt_diloco_outer_f32(ctypes.byref(table), 2, 3, 2, ctypes.byref(sgd), None) == 0
+    assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, 0, ctypes.byref(sgd), None) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

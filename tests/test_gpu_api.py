@@ -22,6 +22,7 @@ from torchft_amd import (
     DiLoCo,
     DistributedDataParallel,
     GradBucketAverager,
+    PureDistributedDataParallel,
     LocalSGD,
     Manager,
     ProcessGroup,
@@ -105,7 +106,7 @@ def peer_world(model, n):
 def test_manager_numerics_generic_process_group(device):
     """torchft/manager_test.py:520-543 on the GPU with a mocked backend: zeroing and
     division are this package's kernels around the backend's (no-op) collective."""
-    m = Manager(pg=create_autospec(ProcessGroup), min_replica_size=2)
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=None, state_dict=None, min_replica_size=2)
     m._quorum_future = MagicMock()
     m._participating_rank, m._participating_world_size = 1, 5
     m._pg.allreduce.return_value = _DummyWork(None)
@@ -129,7 +130,7 @@ def test_manager_allreduce_local_replicas(device, dtype):
     pg = ProcessGroupLocalReplicas(rank=1, world_size=4, peer_participating=[True, True, False])
     pg.register_peers(dev[1], [dev[0], dev[2], dev[3]])
     q = QuorumResult(quorum_id=1, replica_rank=1, replica_world_size=4, max_rank=1, max_world_size=4)
-    m = Manager(pg=pg, min_replica_size=3, world_size_mode=WorldSizeMode.FIXED_WITH_SPARES,
+    m = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=3, world_size_mode=WorldSizeMode.FIXED_WITH_SPARES,
                 quorum_client=Scripted(q))
     m.start_quorum()
     fut = m.allreduce(dev[1])
@@ -148,7 +149,7 @@ def test_manager_allreduce_local_replicas(device, dtype):
 
 def test_manager_error_latch_on_gpu(device):
     pg = ProcessGroupLocalReplicas(rank=0, world_size=2)  # no peers registered
-    m = Manager(pg=pg, min_replica_size=1, quorum_client=StaticQuorum(0, 2))
+    m = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, quorum_client=StaticQuorum(0, 2))
     m.start_quorum()
     t = torch.ones(8, device=device)
     assert m.allreduce(t).wait() is t  # KeyError swallowed
@@ -172,7 +173,7 @@ def test_localsgd_mlp_two_replicas(device):
     for q in peers[0].parameters():
         q.data.add_((torch.randn(q.shape, generator=g) * 1e-3).to(device))
     pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=1e-3)
     with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
         backup0 = cpu(lsgd._backup_parameters.values())
@@ -243,7 +244,7 @@ def test_diloco_fused_local_replicas(device):
             def should_commit(self, rank, step, should_commit, timeout):
                 return should_commit and flag[0]
 
-        return Manager(pg=pg, min_replica_size=1, use_async_quorum=False, quorum_client=Vote(0, 3)), flag
+        return Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, use_async_quorum=False, quorum_client=Vote(0, 3)), flag
 
     m = _run_diloco(device, factory, 3, [True, True, False, True], True)
     assert m.current_step() == 3
@@ -354,7 +355,7 @@ def test_ddp_comm_hook_on_gpu(device):
         return [peer]
 
     pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
-    manager = Manager(pg=pg, min_replica_size=2, quorum_client=StaticQuorum(0, 2))
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, quorum_client=StaticQuorum(0, 2))
     ddp = DistributedDataParallel(manager, model)
     manager.start_quorum()
     ddp(torch.randn(4, 1024, device=device)).square().mean().backward()
@@ -373,6 +374,53 @@ def test_ddp_comm_hook_on_gpu(device):
         for i in bucket:
             assert_bits_equal(params[i].grad.reshape(-1), want[off:off + numels[i]], f"param {i}")
             off += numels[i]
+    manager.shutdown(wait=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pure_ddp_gradients_against_the_checker(device, dtype):
+    """PureDistributedDataParallel (torchft/ddp.py:84-94): one ``manager.allreduce(p.grad)``
+    per parameter from the post-accumulate hook.  Three replicas of which the third is a
+    spare (FIXED_WITH_SPARES, min 2): every gradient must equal the checker's
+    ``manager_allreduce_`` of the three raw gradients with flags [1, 1, 0] and n = 2."""
+    torch.manual_seed(0)
+    model = MLP().to(device=device, dtype=dtype)
+    peers, _ = peer_world(model, 3)
+    for k, peer in enumerate(peers):  # the peers' gradients exist before the local backward
+        peer(torch.randn(4, 1024, device=device, generator=torch.Generator(device).manual_seed(k + 1))
+             .to(dtype)).square().mean().backward()
+    raw = {}
+
+    def lookup(grad):
+        for k, p in enumerate(model.parameters()):
+            if p.grad is not None and p.grad.data_ptr() == grad.data_ptr():
+                raw[k] = grad.detach().cpu().clone()  # the local gradient before averaging
+                return [list(peer.parameters())[k].grad for peer in peers]
+        raise KeyError("unknown tensor")
+
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=3, peer_lookup=lookup,
+                                   peer_participating=[True, False])
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      world_size_mode=WorldSizeMode.FIXED_WITH_SPARES,
+                      quorum_client=StaticQuorum(0, 3))
+    ddp = PureDistributedDataParallel(manager, model)
+    manager.start_quorum()
+    x = torch.randn(4, 1024, device=device, generator=torch.Generator(device).manual_seed(9)).to(dtype)
+    ddp(x).square().mean().backward()
+    torch.cuda.synchronize()
+    assert manager.num_participants() == 2 and manager.is_participating()
+    assert manager.should_commit()
+    params = list(model.parameters())
+    assert sorted(raw) == list(range(len(params)))  # one allreduce per parameter
+    for k, p in enumerate(params):
+        contributions = [raw[k]] + [list(peer.parameters())[k].grad.cpu() for peer in peers]
+        want = O.manager_allreduce_(contributions, [True, True, False], 2, torch.float32)
+        assert_bits_equal(p.grad, want, f"param {k}")
+        if dtype == torch.bfloat16:
+            native = O.manager_allreduce_(contributions, [True, True, False], 2)
+            torch.testing.assert_close(p.grad.cpu().float(), native.float(), rtol=RTOL_BF16, atol=2e-4)
+    # the peers' gradients were only read
+    assert all(q.grad is not None and torch.isfinite(q.grad).all() for peer in peers for q in peer.parameters())
     manager.shutdown(wait=False)
 
 
@@ -559,7 +607,7 @@ def test_diloco_bucketized_on_gpu(device):
     # what the peer contributes to the flat buffer: its pseudo-gradients, back to back
     peer_flat = torch.cat([(q - b).reshape(-1) for q, b in zip(peer_params, backup)]).to(device)
     pg = _PlainLocalPG(lambda t: peer_flat)
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
     inner = optim.SGD(model.parameters(), lr=0.1)
     outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
     with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
@@ -586,7 +634,7 @@ def test_local_sgd_bucketized_on_gpu(device):
     peer_params = [p.data.cpu() + 1e-3 * torch.randn(p.shape) for p in model.parameters()]
     peer_flat = torch.cat([q.reshape(-1) for q in peer_params]).to(device)
     pg = _PlainLocalPG(lambda t: peer_flat)
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=0.1)
     with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
         backup = cpu(lsgd._backup_parameters.values())

@@ -137,22 +137,36 @@ def test_checkpoint_llama3_8b_full_size(device):
         got = (st["exp_avg"].view(torch.int32).sum(dtype=torch.int64).item(),
                st["exp_avg_sq"].view(torch.int32).sum(dtype=torch.int64).item(), int(st["step"]))
         assert got == moments[i], i
-    # views into the staging buffer agree with the scattered copies
+    # every scattered tensor equals the view of the staging buffer it came from (the staging
+    # buffer itself was compared with the source tensors above), element for element
     views = state_pack.unpack(header, staging, copy=False)
     for n, t in out["user"]["model"].items():
-        assert torch.equal(t, views["user"]["model"][n])
-    # PCIe leg on the first 2 GiB of the staging buffer
-    n = 2 << 30
-    host = torch.empty(n, dtype=torch.uint8, pin_memory=True)
-    host.copy_(staging[:n], non_blocking=True)
+        assert torch.equal(t, views["user"]["model"][n]), n
+    for i, st in out["user"]["optim"]["state"].items():
+        ref = views["user"]["optim"]["state"][i]
+        for key in ("exp_avg", "exp_avg_sq", "step"):
+            got, want = st[key], ref[key]
+            assert got.dtype == want.dtype and got.shape == want.shape, (i, key)
+            assert torch.equal(got.view(torch.uint8) if got.dim() else got, 
+                               want.view(torch.uint8) if want.dim() else want), (i, key)
+    del out, views
+    gc.collect()
+    torch.cuda.empty_cache()
+    # the PCIe legs of the configuration: the WHOLE staging buffer to pinned host memory and
+    # back into a second device buffer, through two 1 GiB pinned bounce buffers
+    total = staging.numel()
+    back = torch.empty(total, dtype=torch.uint8, device=device)
+    chunk = 1 << 30
+    bounce = [torch.empty(chunk, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+    for k, lo in enumerate(range(0, total, chunk)):
+        n = min(chunk, total - lo)
+        bounce[k % 2][:n].copy_(staging[lo:lo + n], non_blocking=True)   # same stream: ordered
+        back[lo:lo + n].copy_(bounce[k % 2][:n], non_blocking=True)
     torch.cuda.synchronize()
-    back = torch.empty(n, dtype=torch.uint8, device=device)
-    back.copy_(host, non_blocking=True)
-    torch.cuda.synchronize()
-    assert torch.equal(back, staging[:n])
+    assert torch.equal(back, staging)
 
 
-def test_more_than_2_31_work_items_in_one_launch(device):
+def test_more_than_2_31_work_items_in_one_launch(device, launch_variant):
     """A launch whose slab count exceeds what one grid dimension can hold (40 GiB through
     the byte copy is 5.2 M workgroups of 8 KiB, 10.5 M at 4 KiB) must still cover
     everything: the grid is split in two dimensions."""
@@ -160,11 +174,8 @@ def test_more_than_2_31_work_items_in_one_launch(device):
     src = torch.empty(n, dtype=torch.uint8, device=device)
     src.view(torch.int64).copy_(torch.arange(n // 8, dtype=torch.int64, device=device))
     dst = torch.zeros(n, dtype=torch.uint8, device=device)
-    try:
-        for variant in (1, 2):
-            ops.set_launch_variant(variant)
-            dst.zero_()
-            ops.mt_copy([dst], [src])
-            assert torch.equal(dst, src), f"variant {variant}"
-    finally:
-        ops.set_launch_variant(0)
+    for variant in (1, 2, 1 | (8 << 8)):  # 4 KiB slabs, 8 KiB slabs, 4 KiB with per-XCD runs of 128
+        launch_variant(variant)
+        dst.zero_()
+        ops.mt_copy([dst], [src])
+        assert torch.equal(dst, src), f"variant {variant:#x}"

@@ -215,25 +215,43 @@ def test_mt_copy_mixed_dtypes(device):
         assert_bits_equal(d, s)
 
 
-def test_launch_variants_agree(device):
-    """Every tuning variant computes the same bits."""
+def variant_bits(unroll=0, plain=0, run_log2=None, lds_kib=None):
+    return (unroll | (plain << 4) | ((run_log2 + 1) << 8 if run_log2 is not None else 0)
+            | ((lds_kib // 8 + 1) << 12 if lds_kib is not None else 0))
+
+
+def test_launch_variants_agree(device, launch_variant):
+    """Every launch shape computes the same bits: slab size, plain / non-temporal accesses,
+    per-XCD run length (a permutation of the slab order with a padded grid) and the
+    residency cap."""
     wl = _mlp_workload(2)
     sgd = ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True)
     want = O.diloco_perform_sync(wl.replicas, wl.backup, None, [True, True], 2, True, lr=0.7,
                                  momentum=0.9, nesterov=True)
-    try:
-        for unroll, plain in itertools.product([1, 2, 4], [0, 1]):
-            ops.set_launch_variant(unroll | (plain << 4))
-            b = [t.to(device) for t in wl.backup]
-            m = [torch.empty_like(t) for t in b]
-            p = [torch.empty_like(t) for t in b]
-            reps = [[t.to(device) for t in rep] for rep in wl.replicas]
-            ops.mt_diloco_outer(p, b, m, reps, sgd, True)
-            for i, name in enumerate(wl.names):
-                assert_bits_equal(p[i], want["params"][i], f"variant {unroll}/{plain} {name}")
-                assert_bits_equal(m[i], want["momentum"][i], f"variant {unroll}/{plain} {name}")
-    finally:
-        ops.set_launch_variant(0)
+    shapes = [variant_bits(u, pl) for u, pl in itertools.product([1, 2, 4], [0, 1])]
+    shapes += [variant_bits(u, 0, r, lds) for u in (1, 2, 4) for r, lds in
+               ((0, 0), (3, 0), (6, 64), (7, 32), (12, 0))]
+    for bits in shapes:
+        launch_variant(bits)
+        b = [t.to(device) for t in wl.backup]
+        m = [torch.empty_like(t) for t in b]
+        p = [torch.empty_like(t) for t in b]
+        reps = [[t.to(device) for t in rep] for rep in wl.replicas]
+        ops.mt_diloco_outer(p, b, m, reps, sgd, True)
+        for i, name in enumerate(wl.names):
+            assert_bits_equal(p[i], want["params"][i], f"variant {bits:#x} {name}")
+            assert_bits_equal(b[i], want["backup"][i], f"variant {bits:#x} {name}")
+            assert_bits_equal(m[i], want["momentum"][i], f"variant {bits:#x} {name}")
+        # the flat form and the byte copy take the same shapes
+        x = [torch.randn(300_001, generator=torch.Generator().manual_seed(r)) for r in range(3)]
+        out = torch.empty(300_001, device=device)
+        ops.reduce_avg_(out, [t.to(device) for t in x], 0b101, 2)
+        assert_bits_equal(out, O.manager_allreduce_(x, [True, False, True], 2), f"variant {bits:#x}")
+        src = torch.arange(1_000_003, dtype=torch.int32, device=device).view(torch.uint8)[3:]
+        dst = torch.zeros(src.numel() + 16, dtype=torch.uint8, device=device)
+        ops.mt_copy([dst[7:7 + src.numel()]], [src])
+        assert torch.equal(dst[7:7 + src.numel()], src) and int(dst[:7].sum()) == 0 \
+            and int(dst[7 + src.numel():].sum()) == 0, f"variant {bits:#x}"
 
 
 def test_fp16_rounding_and_overflow(device):
@@ -267,3 +285,158 @@ def test_argument_errors(device):
         ops.reduce_avg_(x.double(), [x.double()])
     with pytest.raises(ValueError):
         ops.reduce_avg_(torch.zeros(4, 4, device=device).t(), [x[:16]])
+
+
+# ---------------------------------------------------------------------------
+# Alignment: a common misalignment of all columns keeps the 128-bit body
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,shift", [(torch.float32, 1), (torch.float32, 3), (torch.bfloat16, 1),
+                                         (torch.bfloat16, 5), (torch.float16, 7)])
+def test_diloco_on_views_behind_an_odd_sized_tensor(device, dtype, shift):
+    """All columns start ``shift`` elements past a 16-byte boundary (what views into flat
+    buffers look like behind an odd-sized tensor): head elements scalar, 128-bit body, scalar
+    tail; several tensors per table, sizes around the slab and head boundaries; guard
+    elements in front of and behind every view must stay untouched."""
+    sizes = [1, 2, 3, 4, 7, 8, 9, 2047, 2048, 2049, 8191, 8192, 8193, 65536 + 3, 300_007]
+    sgd = ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True)
+    g = torch.Generator().manual_seed(11)
+
+    def host(scale):
+        return [(torch.randn(n + shift + 1, generator=g) * scale).to(dtype) for n in sizes]
+
+    backup_h, buf_h = host(0.02), host(1e-3)
+    reps_h = [[(b.float() + 1e-3 * torch.randn(b.shape, generator=g)).to(dtype) for b in backup_h]
+              for _ in range(3)]
+    view = lambda ts: [t[shift:-1] for t in ts]
+    want = O.diloco_perform_sync([view(r) for r in reps_h], view(backup_h), view(buf_h),
+                                 [True, False, True], 2, True, lr=0.7, momentum=0.9, nesterov=True,
+                                 accumulate_dtype=torch.float32)
+    b_d, m_d = [t.to(device) for t in backup_h], [t.to(device) for t in buf_h]
+    p_d = [torch.full_like(t, 7.0) for t in b_d]
+    r_d = [[t.to(device) for t in rep] for rep in reps_h]
+    ops.mt_diloco_outer(view(p_d), view(b_d), view(m_d), [view(r) for r in r_d], sgd, False, 0b101, 2)
+    for i, n in enumerate(sizes):
+        for got, exp, src, what in ((p_d[i], want["params"][i], None, "params"),
+                                    (b_d[i], want["backup"][i], backup_h[i], "backup"),
+                                    (m_d[i], want["momentum"][i], buf_h[i], "momentum")):
+            assert_bits_equal(got[shift:-1], exp, f"{what} n={n}")
+            guard = torch.full((1,), 7.0, dtype=dtype) if src is None else None
+            for sl in (slice(0, shift), slice(-1, None)):
+                assert_bits_equal(got[sl], guard.expand(got[sl].shape) if src is None else src[sl],
+                                  f"{what} guard n={n}")
+        for r in (0, 2):
+            assert_bits_equal(r_d[r][i], reps_h[r][i], f"replica {r} n={n} was modified")
+
+
+@pytest.mark.parametrize("dtype,shift_bytes", [(torch.float32, 4), (torch.bfloat16, 2)])
+def test_large_misaligned_tensor_against_the_checker(device, dtype, shift_bytes):
+    """50 M elements starting 4 bytes (fp32) / 2 bytes (bf16) past a 16-byte boundary, all
+    columns alike: in-place average of three contributions, held to the checker bit for bit
+    (and the same data aligned must give the same values)."""
+    n = 50_000_000
+    shift = shift_bytes // torch.empty(0, dtype=dtype).element_size()
+    g = torch.Generator().manual_seed(3)
+    reps_h = [(torch.randn(n + shift, generator=g) * 0.01).to(dtype) for _ in range(3)]
+    want = O.manager_allreduce_([r[shift:] for r in reps_h], [True, True, True], 3, torch.float32)
+    dev = [r.to(device) for r in reps_h]
+    assert all(d[shift:].data_ptr() % 16 == shift_bytes for d in dev)
+    ops.reduce_avg_(dev[0][shift:], [d[shift:] for d in dev], 0b111, 3)
+    assert_bits_equal(dev[0][shift:], want)
+    assert_bits_equal(dev[0][:shift], reps_h[0][:shift])
+    aligned = [r[shift:].clone().to(device) for r in reps_h]
+    ops.reduce_avg_(aligned[0], aligned, 0b111, 3)
+    assert_bits_equal(aligned[0], want)
+
+
+def test_copy_with_common_and_mixed_misalignment(device):
+    """Byte copy: dst and src misaligned alike (vector body after a head of bytes), alike only
+    modulo 4 (word path), and arbitrarily (byte path); guards around every destination."""
+    g = torch.Generator().manual_seed(5)
+    for n in (1, 5, 15, 16, 17, 4095, 4096, 4097, 70_001, 1_000_003):
+        for d_off, s_off in ((3, 3), (13, 13), (1, 17), (2, 6), (5, 9), (0, 1), (7, 2), (0, 0)):
+            src = torch.randint(0, 256, (n + 64,), dtype=torch.uint8, generator=g)
+            dst = torch.full((n + 64,), 0xAB, dtype=torch.uint8)
+            s_d, d_d = src.to(device), dst.to(device)
+            ops.mt_copy([d_d[d_off:d_off + n]], [s_d[s_off:s_off + n]])
+            want = dst.clone()
+            want[d_off:d_off + n] = src[s_off:s_off + n]
+            assert torch.equal(d_d.cpu(), want), f"n={n} dst+{d_off} src+{s_off}"
+
+
+# ---------------------------------------------------------------------------
+# DiLoCo on bf16 / fp16 parameters (torchft/local_sgd.py:212-215 is dtype-generic)
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sgd_kw", SGD_CASES)
+def test_diloco_16_bit_storage(device, dtype, sgd_kw):
+    """Fused and two-launch forms on 16-bit parameters: fp32 arithmetic, one rounding per
+    stored value.  Bit-exact against the checker's fp32-arithmetic variant; within the stated
+    rtol 1e-2 of the reference form that rounds after every torch op."""
+    wl = _mlp_workload(3)
+    sgd = ops.OuterSGD(**sgd_kw)
+    kw = dict(lr=sgd.lr, momentum=sgd.momentum, dampening=sgd.dampening,
+              weight_decay=sgd.weight_decay, nesterov=sgd.nesterov)
+    flags, mask, nump = [True, True, False], 0b011, 2
+    backup = [t.to(dtype) for t in wl.backup]
+    bufs = None
+    for step in range(2):
+        first = step == 0
+        reps = [[(b.float() + 1e-3 * torch.randn(b.shape, generator=torch.Generator().manual_seed(
+            100 * step + 10 * r + i))).to(dtype) for i, b in enumerate(backup)] for r in range(3)]
+        want = O.diloco_perform_sync(reps, backup, bufs, flags, nump, True, **kw,
+                                     accumulate_dtype=torch.float32)
+        want2 = O.diloco_perform_sync(reps, backup, bufs, flags, nump, True, **kw,
+                                      accumulate_dtype=torch.float32, grads_through_storage=True)
+        native = O.diloco_perform_sync(reps, backup, bufs, flags, nump, True, **kw)
+        to_dev = lambda ts: [t.to(device) for t in ts]
+        for form in ("fused", "two_launch"):
+            b_d, r_d = to_dev(backup), [to_dev(r) for r in reps]
+            m_d = None
+            if sgd.momentum:
+                m_d = [torch.full_like(t, float("nan")) for t in b_d] if first else to_dev(bufs)
+            p_d = r_d[0]  # in place on replica 0, as the API path runs it
+            if form == "fused":
+                ops.mt_diloco_outer(p_d, b_d, m_d, r_d, sgd, first, mask, nump)
+                exp = want
+            else:
+                g_d = [torch.empty_like(t) for t in b_d]
+                ops.mt_pseudograd_avg(g_d, p_d, b_d, r_d, True, mask, nump)
+                for i in range(len(backup)):
+                    assert_bits_equal(g_d[i], want2["grads"][i], f"{form} grads {wl.names[i]}")
+                    assert_bits_equal(p_d[i], backup[i], f"{form} restore {wl.names[i]}")
+                ops.mt_outer_sgd(p_d, b_d, m_d, g_d, sgd, first)
+                exp = want2
+            for i, name in enumerate(wl.names):
+                assert_bits_equal(p_d[i], exp["params"][i], f"{form} step {step} params {name}")
+                assert_bits_equal(b_d[i], exp["backup"][i], f"{form} step {step} backup {name}")
+                if sgd.momentum:
+                    assert_bits_equal(m_d[i], exp["momentum"][i], f"{form} step {step} momentum {name}")
+                    torch.testing.assert_close(m_d[i].cpu().float(), native["momentum"][i].float(),
+                                               rtol=1e-2, atol=2e-4)
+                torch.testing.assert_close(p_d[i].cpu().float(), native["params"][i].float(),
+                                           rtol=1e-2, atol=2e-4)
+        backup, bufs = want["backup"], (want["momentum"] if sgd.momentum else None)
+
+
+def test_fp16_result_is_rounded_from_the_fp32_value(device):
+    """An element whose fp32 result lies exactly on the tie between two fp16 values
+    (0x3a3f5000: the low 13 bits are 0x1000).  The update's last fused multiply-add must
+    first round to fp32 and only then to fp16 (ties to even: 0x11fa); folding both into one
+    mixed-precision instruction rounds the exact product-sum instead and gives 0x11fb."""
+    vals = dict(b=0.001712799072265625, m=0.0012683868408203125, x0=0.0028934478759765625,
+                x2=0.0009288787841796875)
+    n = 5000
+    mk = lambda v: torch.full((n,), v, dtype=torch.float16)
+    b, m, x0, x1, x2 = mk(vals["b"]), mk(vals["m"]), mk(vals["x0"]), mk(123.0), mk(vals["x2"])
+    want = O.diloco_perform_sync([[x0], [x1], [x2]], [b], [m], [True, False, True], 2, True,
+                                 lr=0.7, momentum=0.9, nesterov=True, accumulate_dtype=torch.float32)
+    assert int(want["params"][0][0].view(torch.int16)) == 0x11fa
+    d = lambda t: t.to(device)
+    p_d, b_d, m_d = torch.empty(n, dtype=torch.float16, device=device), d(b), d(m)
+    ops.mt_diloco_outer([p_d], [b_d], [m_d], [[d(x0)], [d(x1)], [d(x2)]],
+                        ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True), False, 0b101, 2)
+    assert_bits_equal(p_d, want["params"][0])
+    assert_bits_equal(b_d, want["backup"][0])
+    assert_bits_equal(m_d, want["momentum"][0])

@@ -90,11 +90,12 @@ def test_concurrent_launches_from_threads(device):
     assert not errors, errors
 
 
-def test_launch_variant_is_thread_local(device):
+def test_launch_variant_is_thread_local(device, launch_variant):
+    """The tuning build's launch-shape override must not leak across threads."""
     seen = {}
 
     def other():
-        ops.set_launch_variant(4 | 16)
+        launch_variant(4 | 16)
         seen["set"] = True
 
     t = threading.Thread(target=other)

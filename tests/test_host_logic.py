@@ -216,8 +216,10 @@ class ScriptedQuorum(QuorumClient):
     def __init__(self, result: QuorumResult) -> None:
         self.result = result
         self.votes = []
+        self.quorum_calls = []
 
     def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+        self.quorum_calls.append(dict(rank=rank, step=step, checkpoint_metadata=checkpoint_metadata))
         return self.result
 
     def should_commit(self, rank, step, should_commit, timeout):
@@ -227,7 +229,7 @@ class ScriptedQuorum(QuorumClient):
 
 def _manager(pg=None, quorum=None, **kw) -> Manager:
     pg = pg if pg is not None else create_autospec(ProcessGroup)
-    return Manager(pg=pg, min_replica_size=kw.pop("min_replica_size", 2),
+    return Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=kw.pop("min_replica_size", 2),
                    quorum_client=quorum or ScriptedQuorum(QuorumResult(
                        quorum_id=123, replica_rank=1, replica_world_size=2, max_step=1,
                        max_rank=1, max_world_size=2)), **kw)
@@ -479,7 +481,7 @@ def test_diloco_fused_on_local_replicas(cpu_ops, commit):
         def should_commit(self, rank, step, should_commit, timeout):
             return should_commit and commit
 
-    manager = Manager(pg=pg, min_replica_size=1, use_async_quorum=False,
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, use_async_quorum=False,
                       quorum_client=Vote(0, 3))
     inner = optim.SGD(model.parameters(), lr=0.1)
     outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
@@ -525,7 +527,7 @@ def test_local_sgd_fused_on_local_replicas(cpu_ops):
         for q in peer.parameters():
             q.data.add_(0.01)
     pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
-    manager = Manager(pg=pg, min_replica_size=1, use_async_quorum=False,
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, use_async_quorum=False,
                       quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=0.1)
     with LocalSGD(manager, model, optimizer, sync_every=1) as local_sgd:
@@ -712,7 +714,7 @@ def test_diloco_bucketized_one_collective_per_sync(cpu_ops):
     torch.manual_seed(0)
     model = SimpleModel()
     pg = _DoublingPG()
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
                       quorum_client=StaticQuorum(0, 2))
     inner = optim.SGD(model.parameters(), lr=0.1)
     outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
@@ -741,7 +743,7 @@ def test_local_sgd_bucketized_one_collective_per_sync(cpu_ops):
     torch.manual_seed(0)
     model = SimpleModel()
     pg = _DoublingPG()
-    manager = Manager(pg=pg, min_replica_size=2, use_async_quorum=False,
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
                       quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=0.1)
     n_total = sum(p.numel() for p in model.parameters())
@@ -771,7 +773,7 @@ def test_manager_client_adapter(cpu_ops):
     peer = MagicMock()
     peer.checkpoint_metadata.return_value = "http://peer/checkpoint/"
     adapter = ManagerClientAdapter(client, connect=lambda address: peer)
-    m = Manager(pg=create_autospec(ProcessGroup), min_replica_size=2, quorum_client=adapter,
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=None, state_dict=None, min_replica_size=2, quorum_client=adapter,
                 timeout=timedelta(seconds=7))
     m._pg.allreduce.return_value = _DummyWork(None)
     m.start_quorum(timeout=timedelta(seconds=12))
@@ -786,3 +788,167 @@ def test_manager_client_adapter(cpu_ops):
     assert adapter.checkpoint_metadata("addr", 3, timedelta(seconds=1)) == "http://peer/checkpoint/"
     peer.checkpoint_metadata.assert_called_once_with(3, timeout=timedelta(seconds=1))
     m.shutdown(wait=False)
+
+
+# ---------------------------------------------------------------------------
+# Manager constructor: the reference's signature (torchft/manager.py:87-108)
+# ---------------------------------------------------------------------------
+
+REFERENCE_MANAGER_PARAMETERS = [
+    # (name, has a default) in the reference's positional order
+    ("pg", False), ("load_state_dict", False), ("state_dict", False), ("min_replica_size", False),
+    ("use_async_quorum", True), ("timeout", True), ("quorum_timeout", True),
+    ("connect_timeout", True), ("rank", True), ("world_size", True), ("world_size_mode", True),
+    ("store_addr", True), ("store_port", True), ("lighthouse_addr", True), ("replica_id", True),
+    ("port", True), ("hostname", True), ("heartbeat_interval", True),
+    ("checkpoint_transport", True),
+]
+
+
+def test_manager_signature_is_the_reference_one():
+    import inspect
+
+    params = list(inspect.signature(Manager.__init__).parameters.values())[1:]
+    positional = [p for p in params if p.kind is p.POSITIONAL_OR_KEYWORD]
+    assert [(p.name, p.default is not p.empty) for p in positional] == REFERENCE_MANAGER_PARAMETERS
+    extra = [p for p in params if p.kind is not p.POSITIONAL_OR_KEYWORD]
+    assert [(p.name, p.kind) for p in extra] == [("quorum_client", inspect.Parameter.KEYWORD_ONLY)]
+    assert inspect.signature(Manager.__init__).parameters["use_async_quorum"].default is True
+    assert inspect.signature(Manager.__init__).parameters["timeout"].default == timedelta(seconds=60)
+
+
+def test_manager_constructed_like_the_reference_integration_test(monkeypatch):
+    """The call of torchft/manager_integ_test.py:148-161 binds; without a quorum client it is
+    refused with one clear error (the control plane is not part of this package), with one
+    it builds a manager that carries the reference's default checkpoint transport."""
+    monkeypatch.delenv("TORCHFT_LIGHTHOUSE", raising=False)
+    pg = create_autospec(ProcessGroup)
+    kwargs = dict(
+        pg=pg, min_replica_size=2, load_state_dict=lambda sd: None, state_dict=lambda: {},
+        replica_id="0", store_addr="localhost", store_port=29500, rank=0, world_size=1,
+        lighthouse_addr="http://localhost:29510", port=19530,
+    )
+    with pytest.raises(NotImplementedError, match="control plane not built; pass quorum_client="):
+        Manager(**kwargs)
+    quorum = ScriptedQuorum(QuorumResult(quorum_id=1, replica_rank=0, replica_world_size=2,
+                                         max_step=0, max_rank=0, max_world_size=2))
+    m = Manager(**kwargs, quorum_client=quorum, use_async_quorum=False)
+    try:
+        assert isinstance(m._checkpoint_transport, CheckpointServer)
+        m.start_quorum()
+        assert m.num_participants() == 2 and m.is_participating()
+        assert quorum.quorum_calls[0]["checkpoint_metadata"].startswith("http://")
+    finally:
+        m.shutdown(wait=False)
+
+
+def test_manager_constructed_like_train_ddp(monkeypatch):
+    """The call of train_ddp.py:82-89 (everything else from the environment)."""
+    monkeypatch.delenv("TORCHFT_LIGHTHOUSE", raising=False)
+    monkeypatch.setenv("RANK", "0")
+    pg = create_autospec(ProcessGroup)
+    pg.size.return_value = 1
+    kwargs = dict(pg=pg, min_replica_size=1, load_state_dict=lambda sd: None, state_dict=lambda: {},
+                  replica_id="train_ddp_0", timeout=timedelta(seconds=10))
+    m = Manager(**kwargs)
+    m.start_quorum()
+    m.wait_quorum()
+    assert m.num_participants() == 1 and m._rank == 0 and m._timeout == timedelta(seconds=10)
+    m.shutdown(wait=False)
+    monkeypatch.setenv("TORCHFT_LIGHTHOUSE", "http://lighthouse:29510")
+    with pytest.raises(NotImplementedError, match="control plane not built"):
+        Manager(**kwargs)
+    # positional, in the reference's order
+    m = Manager(pg, None, None, 1, False, timedelta(seconds=5), timedelta(seconds=6),
+                timedelta(seconds=7), 3, 4, WorldSizeMode.FIXED_WITH_SPARES, None, None, None, "r",
+                None, "host", timedelta(milliseconds=50), None, quorum_client=StaticQuorum(0, 1))
+    assert (m._rank, m._use_async_quorum, m._world_size_mode) == (3, False, WorldSizeMode.FIXED_WITH_SPARES)
+    assert (m._timeout, m._quorum_timeout, m._connect_timeout) == (
+        timedelta(seconds=5), timedelta(seconds=6), timedelta(seconds=7))
+    m.shutdown(wait=False)
+
+
+def test_local_sgd_fused_waits_for_an_asynchronous_quorum(cpu_ops):
+    """LocalSGD allows ``use_async_quorum=True`` (the Manager's default).  The single-launch
+    sync decides before it reduces, so it must join the quorum thread first: otherwise the
+    vote reads the previous quorum's participant count (0 before the first one, so no
+    commit) and a recovered state is not applied (torchft/manager.py:265 reaches
+    ``wait_quorum`` through ``allreduce`` before ``should_commit``)."""
+    import time
+
+    torch.manual_seed(3)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 2)
+    for peer in peers:
+        for q in peer.parameters():
+            q.data.add_(0.01)
+
+    class SlowQuorum(StaticQuorum):
+        def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+            time.sleep(0.3)
+            return super().quorum(rank, step, checkpoint_metadata, shrink_only, timeout)
+
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    client = SlowQuorum(0, 2)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      use_async_quorum=True, quorum_client=client)
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1) as local_sgd:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.grad = torch.zeros_like(p)
+        local = [p.data.clone() for p in model.parameters()]
+        want = O.localsgd_perform_sync(
+            [local, [q.data.clone() for q in peers[0].parameters()]],
+            [b.clone() for b in local_sgd._backup_parameters.values()], [True, True], 2, True)
+        optimizer.step()  # first sync: quorum still running when the sync starts
+        assert client.commit_votes == [True]
+        assert manager.current_step() == 1 and manager.batches_committed() == 2
+        for p, w in zip(model.parameters(), want["params"]):
+            assert_bits_equal(p.data, w)
+        assert cpu_ops.calls.count("mt_reduce_avg") == 1
+    manager.shutdown(wait=False)
+
+
+def test_local_sgd_fused_applies_recovered_state_with_asynchronous_quorum(cpu_ops):
+    """A healing replica under an asynchronous quorum: the pending state dict is loaded by
+    the vote (torchft/manager.py:572-575), the replica does not participate, and its
+    parameters end as the average of the others."""
+    import time
+
+    torch.manual_seed(4)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 2)
+    loaded = []
+
+    class HealingQuorum(QuorumClient):
+        def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+            time.sleep(0.2)
+            return QuorumResult(quorum_id=7, replica_rank=0, replica_world_size=2,
+                                recover_src_manager_address="peer", recover_src_rank=1,
+                                max_step=5, max_rank=None, max_world_size=1, heal=True)
+
+        def should_commit(self, rank, step, should_commit, timeout):
+            return should_commit
+
+        def checkpoint_metadata(self, address, rank, timeout):
+            return "meta"
+
+    transport = MagicMock()
+    transport.metadata.return_value = ""
+    transport.recv_checkpoint.return_value = {"user": {"tag": 1}, "torchft": {"step": 5, "batches_committed": 10}}
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    manager = Manager(pg=pg, load_state_dict=loaded.append, state_dict=lambda: {}, min_replica_size=1,
+                      use_async_quorum=True, quorum_client=HealingQuorum(), checkpoint_transport=transport)
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1):
+        with torch.no_grad():
+            for p in model.parameters():
+                p.grad = torch.zeros_like(p)
+        optimizer.step()
+        assert loaded == [{"tag": 1}]
+        assert manager.current_step() == 6
+        # not participating: contributes zeros, one participant -> the peer's values
+        for p, q in zip(model.parameters(), peers[0].parameters()):
+            assert_bits_equal(p.data, q.data)
+    manager.shutdown(wait=False)

@@ -41,7 +41,53 @@ def _assert_models_equal(results):
             assert_bits_equal(state[k], state0[k], k)
 
 
+def _assert_syncs_match_the_checker(results, kind):
+    """Every synchronisation the cluster ran, held to the CPU checker: the recorded inputs of
+    all replicas of a quorum (parameters after the inner steps, shared backup, outer momentum)
+    go through ``O.diloco_perform_sync`` / ``O.localsgd_perform_sync`` and every participating
+    replica's recorded outputs must equal the result bit for bit
+    (torchft/manager_integ_test.py:553-562 asserts only that replicas agree with each other)."""
+    from oracle import replica_sync as O
+
+    by_step = {}
+    for _, _, records in results:
+        for rec in records:
+            by_step.setdefault(rec["step"], {})[rec["rank"]] = rec
+    checked = 0
+    for step, ranks in sorted(by_step.items()):
+        world = next(iter(ranks.values()))["world"]
+        if sorted(ranks) != list(range(world)) or any(r["world"] != world for r in ranks.values()):
+            continue  # a replica died before this sync: the others latched an error or re-formed
+        recs = [ranks[r] for r in range(world)]
+        flags = [r["participating"] for r in recs]
+        if not any(flags):
+            continue
+        src = recs[flags.index(True)]
+        nump = src["num_participants"]
+        assert all(r["num_participants"] == nump for r in recs)
+        commit = src["committed"]
+        assert all(r["committed"] == commit for r in recs)
+        reps = [r["params"] for r in recs]
+        if kind == "diloco":
+            want = O.diloco_perform_sync(reps, src["backup"], src["momentum"], flags, nump, commit,
+                                         lr=0.7, momentum=0.9, nesterov=True)
+        else:
+            want = O.localsgd_perform_sync(reps, src["backup"], flags, nump, commit)
+        for rec, part in zip(recs, flags):
+            if not part:
+                continue  # a healing replica ends with the recovered state, checked elsewhere
+            for t in range(len(want["params"])):
+                assert_bits_equal(rec["post_params"][t], want["params"][t], f"step {step} params[{t}]")
+                assert_bits_equal(rec["post_backup"][t], want["backup"][t], f"step {step} backup[{t}]")
+                if kind == "diloco" and commit:
+                    assert_bits_equal(rec["post_momentum"][t], want["momentum"][t],
+                                      f"step {step} momentum[{t}]")
+            checked += 1
+    assert checked >= 4, f"only {checked} replica-syncs could be held to the checker"
+
+
 def _assert_histories_equal(results, check_momentum):
+    results = [(r[0], r[1]) for r in results]
     (hist0, step0), *rest = results
     assert step0 >= 4
     for hist, step in rest:
@@ -76,6 +122,7 @@ def test_local_sgd_recovery(dev):
     injectors = [H.FailureInjector(), H.FailureInjector().fail_at(1, 2)]
     results = H.run_cluster(H.local_sgd_train_loop, dev, injectors)
     _assert_histories_equal(results, check_momentum=False)
+    _assert_syncs_match_the_checker(results, "local_sgd")
     assert injectors[1].count == 1
 
 
@@ -84,6 +131,7 @@ def test_diloco_healthy(dev):
     results = H.run_cluster(H.diloco_train_loop, dev, [H.FailureInjector(), H.FailureInjector()],
                             use_async_quorum=False)
     _assert_histories_equal(results, check_momentum=True)
+    _assert_syncs_match_the_checker(results, "diloco")
 
 
 @pytest.mark.parametrize("cpu_ops_if_cpu", _devices(), indirect=True)
@@ -91,6 +139,7 @@ def test_diloco_recovery(dev):
     injectors = [H.FailureInjector(), H.FailureInjector().fail_at(1, 2)]
     results = H.run_cluster(H.diloco_train_loop, dev, injectors, use_async_quorum=False)
     _assert_histories_equal(results, check_momentum=True)
+    _assert_syncs_match_the_checker(results, "diloco")
     assert injectors[1].count == 1
 
 
@@ -148,7 +197,7 @@ def test_thread_process_group_masks_and_missing_peer(cpu_ops):
     commits = [None] * 3
 
     def replica(r, quorum_id, show_up=True, timeout=5.0):
-        m = Manager(pg=ProcessGroupThreads(world), min_replica_size=2,
+        m = Manager(pg=ProcessGroupThreads(world), load_state_dict=None, state_dict=None, min_replica_size=2,
                     timeout=timedelta(seconds=timeout), quorum_client=Fixed(r, quorum_id))
         m.start_quorum(allow_heal=False)
         if show_up:

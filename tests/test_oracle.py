@@ -209,6 +209,57 @@ def test_diloco_reference_loop_matches_restatement():
             p.data.copy_(r)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_diloco_fp32_arithmetic_for_16_bit_storage(dtype):
+    """The fp32-arithmetic variant for bf16 / fp16 parameters (what the kernels compute):
+    (1) for values that are exact in the storage dtype the whole step evaluated in float64
+    and rounded once differs from it by at most one unit in the last place of the storage
+    dtype (fp32 error is far below half a 16-bit ulp, so only ties can differ);
+    (2) it stays within the stated rtol 1e-2 (atol for near-zero values) of the reference
+    form, where torch rounds to the storage dtype after every op
+    (torchft/local_sgd.py:212-215 on bf16 parameters);
+    (3) passing the averaged pseudo-gradient through memory in the storage dtype (the
+    two-launch form) changes results by no more than that same tolerance."""
+    shapes = [("w", (257, 5)), ("b", (9,))]
+    wl = workloads.make_diloco_workload(shapes, 3, torch.device("cpu"))
+    backup = [t.to(dtype) for t in wl.backup]
+    reps = [[t.to(dtype) for t in rep] for rep in wl.replicas]
+    bufs = [(1e-3 * torch.randn(t.shape, generator=torch.Generator().manual_seed(5))).to(dtype)
+            for t in backup]
+    flags, nump = [True, True, False], 2
+    kw = dict(lr=0.7, momentum=0.9, nesterov=True)
+    for first in (True, False):
+        mb = None if first else bufs
+        got = O.diloco_perform_sync(reps, backup, mb, flags, nump, True, **kw,
+                                    accumulate_dtype=torch.float32)
+        native = O.diloco_perform_sync(reps, backup, mb, flags, nump, True, **kw)
+        two = O.diloco_perform_sync(reps, backup, mb, flags, nump, True, **kw,
+                                    accumulate_dtype=torch.float32, grads_through_storage=True)
+        for t, b in enumerate(backup):
+            assert got["params"][t].dtype == dtype and got["momentum"][t].dtype == dtype
+            # (1) float64 evaluation of the same formulas
+            b64 = b.double()
+            g64 = sum((rep[t].double() - b64) for rep, f in zip(reps, flags) if f) / nump
+            buf64 = g64 if first else 0.9 * bufs[t].double() + g64
+            p64 = b64 - 0.7 * (g64 + 0.9 * buf64)
+            for name, exact in (("params", p64), ("backup", p64), ("momentum", buf64), ("grads", g64)):
+                rounded = exact.to(dtype)
+                ulp_apart = (got[name][t].view(torch.int16).int() - rounded.view(torch.int16).int()).abs()
+                assert int(ulp_apart.max()) <= 1, (name, first)
+                assert float((ulp_apart > 0).float().mean()) < 0.02, (name, first)
+            # (2) and (3)
+            for name in ("params", "backup", "momentum", "grads"):
+                torch.testing.assert_close(got[name][t].float(), native[name][t].float(), rtol=1e-2, atol=2e-4)
+                torch.testing.assert_close(got[name][t].float(), two[name][t].float(), rtol=1e-2, atol=2e-4)
+    # fp32 storage: the option changes nothing
+    a = O.diloco_perform_sync(wl.replicas, wl.backup, None, flags, nump, True, **kw)
+    b_ = O.diloco_perform_sync(wl.replicas, wl.backup, None, flags, nump, True, **kw,
+                               accumulate_dtype=torch.float32, grads_through_storage=True)
+    for name in ("params", "backup", "momentum", "grads"):
+        for x, y in zip(a[name], b_[name]):
+            assert_bits_equal(x, y)
+
+
 def test_localsgd_closed_form_and_invariants():
     wl = _tiny_workload(2)
     res = O.localsgd_perform_sync(wl.replicas, wl.backup, [True, True], 2, True)

@@ -18,7 +18,7 @@ import torch  # noqa: F401  (must precede loading the library, see module docstr
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchft_amd.so"
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 MAX_REPLICAS = 8
 MIN_CHUNK_ELEMS = 8192
 MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
@@ -69,17 +69,16 @@ SIGNATURES = {
         c_int,
         [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_uint32, c_int, c_void_p],
     ),
-    "tft_mt_diloco_outer_f32": (
+    "tft_mt_diloco_outer": (
         c_int,
-        [POINTER(MtTable), c_uint32, c_uint32, c_uint32, POINTER(SgdParams), c_void_p],
+        [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_int, POINTER(SgdParams), c_void_p],
     ),
-    "tft_mt_pseudograd_avg_f32": (
+    "tft_mt_pseudograd_avg": (
         c_int,
-        [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_int, c_void_p],
+        [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_int, c_int, c_void_p],
     ),
-    "tft_mt_outer_sgd_f32": (c_int, [POINTER(MtTable), POINTER(SgdParams), c_void_p]),
+    "tft_mt_outer_sgd": (c_int, [POINTER(MtTable), c_int, POINTER(SgdParams), c_void_p]),
     "tft_mt_copy_bytes": (c_int, [POINTER(MtTable), c_void_p]),
-    "tft_set_launch_variant": (None, [c_uint32]),
 }
 
 
@@ -107,36 +106,40 @@ def _check_single_hip_runtime() -> None:
         )
 
 
+def load(path: Path, extra_signatures: Optional[dict] = None) -> ctypes.CDLL:
+    """Loads a build of the library from ``path`` and binds every declared symbol."""
+    if not path.exists():
+        raise NativeLibraryError(
+            f"{path} is not built; run `python -m torchft_amd._build` "
+            "(needs hipcc, cross-compiles for gfx950 without a GPU)"
+        )
+    try:
+        handle = ctypes.CDLL(str(path), mode=ctypes.RTLD_LOCAL)
+    except OSError as e:
+        raise NativeLibraryError(f"cannot load {path}: {e}") from e
+    for name, (restype, argtypes) in {**SIGNATURES, **(extra_signatures or {})}.items():
+        try:
+            fn = getattr(handle, name)
+        except AttributeError as e:
+            raise NativeLibraryError(f"{path} does not export {name}") from e
+        fn.restype = restype
+        fn.argtypes = argtypes
+    version = handle.tft_abi_version()
+    if version != ABI_VERSION:
+        raise NativeLibraryError(f"ABI version {version}, this package expects {ABI_VERSION}")
+    _check_single_hip_runtime()
+    return handle
+
+
 def lib() -> ctypes.CDLL:
     """Returns the loaded library; raises NativeLibraryError if it cannot be loaded."""
     global _lib
     if _lib is not None:
         return _lib
     with _lock:
-        if _lib is not None:
-            return _lib
-        if not LIB_PATH.exists():
-            raise NativeLibraryError(
-                f"{LIB_PATH} is not built; run `python -m torchft_amd._build` "
-                "(needs hipcc, cross-compiles for gfx950 without a GPU)"
-            )
-        try:
-            handle = ctypes.CDLL(str(LIB_PATH), mode=ctypes.RTLD_LOCAL)
-        except OSError as e:
-            raise NativeLibraryError(f"cannot load {LIB_PATH}: {e}") from e
-        for name, (restype, argtypes) in SIGNATURES.items():
-            try:
-                fn = getattr(handle, name)
-            except AttributeError as e:
-                raise NativeLibraryError(f"{LIB_PATH} does not export {name}") from e
-            fn.restype = restype
-            fn.argtypes = argtypes
-        version = handle.tft_abi_version()
-        if version != ABI_VERSION:
-            raise NativeLibraryError(f"ABI version {version}, this package expects {ABI_VERSION}")
-        _check_single_hip_runtime()
-        _lib = handle
-        return handle
+        if _lib is None:
+            _lib = load(LIB_PATH)
+        return _lib
 
 
 def check(rc: int, what: str) -> None:

@@ -21,6 +21,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <string.h>
 
 #include "torchft_amd.h"
 
@@ -32,7 +33,9 @@ constexpr int kMaxCols = TFT_MAX_REPLICAS + 3;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 thread_local char g_err[512] = "";
-thread_local uint32_t g_variant = 0;
+#ifdef TFT_TUNING
+thread_local uint32_t g_variant = 0;  // tuning builds only: overrides the launch shape
+#endif
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -97,7 +100,12 @@ struct F16 {
   static constexpr int kVec = 8;
   __device__ static inline float widen1(uint16_t x) { return __half2float(__ushort_as_half(x)); }
   __device__ static inline uint16_t narrow1(float x) {
-    return __half_as_ushort(__float2half_rn(x));  // round to nearest even
+    // The fp32 value is final before it is converted.  Without this barrier the
+    // compiler folds a preceding fused multiply-add and the conversion into one
+    // v_fma_mixlo_f16, which rounds the exact product-sum to fp16 directly and so
+    // differs from "fp32 result, then round to nearest even" on (near-)ties.
+    asm volatile("" : "+v"(x));
+    return __half_as_ushort(__float2half_rn(x));
   }
   __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
 #pragma unroll
@@ -135,10 +143,19 @@ __device__ inline void store16(void* p, const u32x4& v) {
 // A launch of more than 2^31 work-items in one grid dimension is silently cut
 // short by the runtime, so large slab counts are laid out as a 2-D grid with a
 // bounded x extent (see grid_for); the dispatcher still hands workgroups out
-// x-fastest, i.e. in slab order.
+// x-fastest, i.e. in workgroup-id order.
 constexpr uint32_t kMaxGridX = 1u << 22;
+constexpr uint32_t kMaxRunLog2 = 12;  // longest per-XCD run: 4096 slabs
 
-__device__ inline uint32_t slab_index() { return blockIdx.y * gridDim.x + blockIdx.x; }
+// Workgroup id -> slab.  Ids go round-robin over the 8 XCDs; XCD x takes the
+// x-th run of 2^run_log2 consecutive slabs out of every group of 8 runs.
+__device__ inline uint32_t slab_index(uint32_t run_log2) {
+  const uint32_t id = blockIdx.y * gridDim.x + blockIdx.x;
+  const uint32_t xcd = id & 7u, j = id >> 3;
+  const uint32_t within = j & ((1u << run_log2) - 1u), group = j >> run_log2;
+  return (((group << 3) + xcd) << run_log2) + within;
+}
+
 struct TableArgs {
   void* const* ptrs;
   const uint64_t* numel;
@@ -148,49 +165,88 @@ struct TableArgs {
   uint32_t chunk_elems;
   uint32_t slab_shift;  // log2(slabs per chunk)
   uint32_t total_chunks;
+  uint32_t run_log2;
 };
 
 struct FlatArgs {  // one tensor, pointers carried in the kernel arguments
   void* ptrs[kMaxCols];
   uint64_t numel;
+  uint32_t run_log2;
 };
 
-// Both return the number of elements of this workgroup's slab (0: nothing to do).
+// What one workgroup has to do: `n` elements starting at ptr, with 128-bit
+// accesses if `vec`; the first slab of a misaligned tensor also has a head, the
+// `head` elements starting at ptr - shift (the tensor's first elements, up to the
+// 16-byte boundary or the tensor's end), done with scalar accesses.
+struct SlabWork {
+  uint32_t n;
+  uint32_t head;
+  uint32_t shift;  // elements from the tensor's base to the first aligned one
+  bool vec;
+};
+
+// Shared by both locators: given the tensor's column base pointers, the slab's
+// ordinal k inside the tensor and the tensor's size, computes the work and
+// advances the active pointers to the first body element.
+template <int NCOL>
+__device__ inline SlabWork place_slab(char* (&ptr)[NCOL], uint32_t cols, uint64_t numel, uint64_t k,
+                                      uint32_t slab_elems, uint32_t esize) {
+  // common misalignment of the active columns (the shift keeps them aligned together)
+  uint32_t mis = 0xffffffffu;
+  bool same = true;
+#pragma unroll
+  for (int c = 0; c < NCOL; ++c) {
+    if ((cols >> c) & 1u) {
+      const uint32_t m = (uint32_t)(reinterpret_cast<uintptr_t>(ptr[c]) & 15u);
+      if (mis == 0xffffffffu) mis = m;
+      same = same && (m == mis);
+    }
+  }
+  SlabWork w;
+  w.vec = same && (mis % esize == 0);
+  const uint32_t h = w.vec ? ((16u - mis) & 15u) / esize : 0u;  // elements up to the boundary
+  const uint64_t begin = k * slab_elems + h;
+  w.shift = h;
+  w.head = (k == 0) ? (uint32_t)(numel < h ? numel : h) : 0u;
+  w.n = 0;
+  if (begin < numel) {
+    const uint64_t left = numel - begin;
+    w.n = left < slab_elems ? (uint32_t)left : slab_elems;
+  }
+#pragma unroll
+  for (int c = 0; c < NCOL; ++c)
+    ptr[c] = ((cols >> c) & 1u) ? ptr[c] + begin * esize : nullptr;
+  return w;
+}
+
 template <int NCOL>
 struct TableLocator {
   typedef TableArgs args_t;
-  __device__ static inline uint32_t locate(const TableArgs& a, uint32_t slab, uint32_t slab_elems,
-                                           uint32_t cols, char* (&ptr)[NCOL], size_t esize) {
+  __device__ static inline SlabWork locate(const TableArgs& a, uint32_t slab_elems, uint32_t cols,
+                                           char* (&ptr)[NCOL], uint32_t esize) {
+    const uint32_t slab = slab_index(a.run_log2);
     const uint32_t chunk = slab >> a.slab_shift;
-    if (chunk >= a.total_chunks) return 0;  // padding of the 2-D grid
+    if (chunk >= a.total_chunks) return SlabWork{0, 0, 0, false};  // padding of the grid
     const uint32_t sub = slab & ((1u << a.slab_shift) - 1u);
     const uint32_t t = a.chunk_tensor[chunk];
     const uint64_t numel = a.numel[t];
-    const uint64_t base =
-        (uint64_t)(chunk - a.chunk_start[t]) * a.chunk_elems + (uint64_t)sub * slab_elems;
-    if (base >= numel) return 0;
+    const uint64_t k = ((uint64_t)(chunk - a.chunk_start[t]) << a.slab_shift) + sub;
 #pragma unroll
     for (int c = 0; c < NCOL; ++c)
-      ptr[c] = ((cols >> c) & 1u)
-                   ? static_cast<char*>(a.ptrs[(size_t)c * a.n_tensors + t]) + base * esize
-                   : nullptr;
-    const uint64_t left = numel - base;
-    return left < slab_elems ? (uint32_t)left : slab_elems;
+      ptr[c] = ((cols >> c) & 1u) ? static_cast<char*>(a.ptrs[(size_t)c * a.n_tensors + t]) : nullptr;
+    return place_slab<NCOL>(ptr, cols, numel, k, slab_elems, esize);
   }
 };
 
 template <int NCOL>
 struct FlatLocator {
   typedef FlatArgs args_t;
-  __device__ static inline uint32_t locate(const FlatArgs& a, uint32_t slab, uint32_t slab_elems,
-                                           uint32_t cols, char* (&ptr)[NCOL], size_t esize) {
-    const uint64_t base = (uint64_t)slab * slab_elems;
-    if (base >= a.numel) return 0;
+  __device__ static inline SlabWork locate(const FlatArgs& a, uint32_t slab_elems, uint32_t cols,
+                                           char* (&ptr)[NCOL], uint32_t esize) {
+    const uint64_t k = slab_index(a.run_log2);  // slabs past the end get n = 0 from place_slab
 #pragma unroll
-    for (int c = 0; c < NCOL; ++c)
-      ptr[c] = ((cols >> c) & 1u) ? static_cast<char*>(a.ptrs[c]) + base * esize : nullptr;
-    const uint64_t left = a.numel - base;
-    return left < slab_elems ? (uint32_t)left : slab_elems;
+    for (int c = 0; c < NCOL; ++c) ptr[c] = ((cols >> c) & 1u) ? static_cast<char*>(a.ptrs[c]) : nullptr;
+    return place_slab<NCOL>(ptr, cols, a.numel, k, slab_elems, esize);
   }
 };
 
@@ -273,25 +329,28 @@ __global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_
   constexpr int NCOL = Op::NCOL;
   constexpr int V = E::kVec;
   constexpr uint32_t kSlab = kThreads * V * U;
+  constexpr uint32_t kEsize = sizeof(typename E::elem_t);
   const uint32_t rmask = op.rmask();
   const uint32_t wmask = op.wmask();
   char* ptr[NCOL];
-  const uint32_t n =
-      Loc::locate(args, slab_index(), kSlab, rmask | wmask, ptr, sizeof(typename E::elem_t));
-  if (n == 0) return;
-  uintptr_t bits = 0;
+  const SlabWork w = Loc::locate(args, kSlab, rmask | wmask, ptr, kEsize);
+  if (w.head) {  // first slab of a misaligned tensor: the elements before the boundary
+    char* hp[NCOL];
 #pragma unroll
-  for (int c = 0; c < NCOL; ++c) bits |= reinterpret_cast<uintptr_t>(ptr[c]);
-  if ((bits & 15u) == 0) {
-    if (n == kSlab) {
+    for (int c = 0; c < NCOL; ++c) hp[c] = ptr[c] ? ptr[c] - (size_t)w.shift * kEsize : nullptr;
+    scalar_range<E, Op>(hp, op, 0, w.head, rmask, wmask);
+  }
+  if (w.n == 0) return;
+  if (w.vec) {
+    if (w.n == kSlab) {
       stream_block<E, Op, U, NT, false>(ptr, op, 0, kSlab / V, rmask, wmask);
     } else {
-      const uint32_t nvec = n / V;
+      const uint32_t nvec = w.n / V;
       if (nvec) stream_block<E, Op, U, NT, true>(ptr, op, 0, nvec, rmask, wmask);
-      if (nvec * V < n) scalar_range<E, Op>(ptr, op, nvec * V, n, rmask, wmask);
+      if (nvec * V < w.n) scalar_range<E, Op>(ptr, op, nvec * V, w.n, rmask, wmask);
     }
   } else {
-    scalar_range<E, Op>(ptr, op, 0, n, rmask, wmask);
+    scalar_range<E, Op>(ptr, op, 0, w.n, rmask, wmask);
   }
 }
 
@@ -420,13 +479,17 @@ template <int U, bool NT>
 __global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {
   constexpr uint32_t kSlab = kThreads * 16 * U;  // bytes
   char* ptr[2];
-  const uint32_t n = TableLocator<2>::locate(args, slab_index(), kSlab, 3u, ptr, 1);
-  if (n == 0) return;
+  // esize 1: place_slab shifts the slabs to the common 16-byte boundary of dst and src
+  const SlabWork w = TableLocator<2>::locate(args, kSlab, 3u, ptr, 1);
   char* dst = ptr[0];
   char* src = ptr[1];
-  const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+  if (w.head) {
+    for (uint32_t i = threadIdx.x; i < w.head; i += kThreads) (dst - w.shift)[i] = (src - w.shift)[i];
+  }
+  if (w.n == 0) return;
+  const uint32_t n = w.n;
   uint32_t done = 0;
-  if ((bits & 15u) == 0) {
+  if (w.vec) {
     const uint32_t nvec = n / 16;
     if (NT) {
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(src, 0, nvec * 16, kBufferWord3);
@@ -447,31 +510,66 @@ __global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {
         store16<false>(dst + (size_t)v * 16, load16<false>(src + (size_t)v * 16));
     }
     done = nvec * 16;
-  } else if ((bits & 3u) == 0) {
-    const uint32_t nw = n / 4;
-    for (uint32_t w = threadIdx.x; w < nw; w += kThreads)
-      reinterpret_cast<uint32_t*>(dst)[w] = reinterpret_cast<const uint32_t*>(src)[w];
-    done = nw * 4;
+  } else {
+    // dst and src are misaligned differently: widest access both sides allow
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) ^ reinterpret_cast<uintptr_t>(src);
+    if ((bits & 3u) == 0) {
+      // bytes up to dst's 4-byte boundary, then words
+      const uint32_t lead = (4u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 3u)) & 3u;
+      const uint32_t pre = lead < n ? lead : n;
+      if (threadIdx.x < pre) dst[threadIdx.x] = src[threadIdx.x];
+      const uint32_t nw = (n - pre) / 4;
+      for (uint32_t i = threadIdx.x; i < nw; i += kThreads)
+        reinterpret_cast<uint32_t*>(dst + pre)[i] = reinterpret_cast<const uint32_t*>(src + pre)[i];
+      done = pre + nw * 4;
+    }
   }
   for (uint32_t i = done + threadIdx.x; i < n; i += kThreads) dst[i] = src[i];
 }
 
 // ---------------------------------------------------------------------------
-// Host side: validation and dispatch.
+// Host side: validation, launch shape and dispatch.
 // ---------------------------------------------------------------------------
-struct Variant {
-  int unroll;  // 128-bit accesses per lane and stream: 1, 2 or 4
+
+// How a kernel is launched: 128-bit accesses per lane and stream (slab size in
+// units of 4 KiB), per-XCD run length, unused dynamic LDS to cap residency.
+struct Shape {
+  int unroll;
   bool nt;
+  uint32_t run_log2;
+  uint32_t lds_bytes;
 };
 
-// default_unroll: slab size (in 4 KiB units per stream) that measured best for the
-// calling kernel on MI355X; the thread's launch variant overrides it.
-Variant decode_variant(int default_unroll) {
-  Variant v{default_unroll, true};
-  const uint32_t bits = g_variant;
-  if ((bits & 0xfu) == 1 || (bits & 0xfu) == 2 || (bits & 0xfu) == 4) v.unroll = (int)(bits & 0xfu);
-  if (bits & 0x10u) v.nt = false;
-  return v;
+enum Family { kFamReduce, kFamDiloco, kFamPseudograd, kFamOuterSgd, kFamCopy };
+
+// Tuned on MI355X.  `traffic` is the launch's algorithmic bytes: launches that
+// move less than a few GB finish in under a millisecond and are dominated by the
+// ramp and tail of the in-flight window, which a residency cap of two workgroups
+// per CU and short per-XCD runs shorten; large launches want the widest window.
+Shape pick_shape(Family fam, uint64_t traffic) {
+  Shape s{2, true, 0, 0};
+  const bool small = traffic < (16ull << 30);
+  switch (fam) {
+    case kFamReduce: s.unroll = 4; break;
+    case kFamDiloco: s.unroll = small ? 2 : 1; break;
+    case kFamPseudograd: s.unroll = 2; break;
+    case kFamOuterSgd: s.unroll = 2; break;
+    case kFamCopy: s.unroll = 1; break;
+  }
+  if (small && fam != kFamCopy) {
+    s.run_log2 = 6;
+    s.lds_bytes = 64u << 10;
+  }
+#ifdef TFT_TUNING
+  // bits 0-3 unroll (1, 2, 4), bit 4 plain accesses, bits 8-11 run_log2 + 1,
+  // bits 12-15 LDS bytes / 8 KiB + 1; a zero field keeps the default
+  const uint32_t v = g_variant;
+  if ((v & 0xfu) == 1 || (v & 0xfu) == 2 || (v & 0xfu) == 4) s.unroll = (int)(v & 0xfu);
+  if (v & 0x10u) s.nt = false;
+  if ((v >> 8) & 0xfu) s.run_log2 = ((v >> 8) & 0xfu) - 1;
+  if ((v >> 12) & 0xfu) s.lds_bytes = (((v >> 12) & 0xfu) - 1) * 8192u;
+#endif
+  return s;
 }
 
 bool is_pow2(uint32_t x) { return x && !(x & (x - 1)); }
@@ -482,12 +580,6 @@ uint32_t log2u(uint32_t x) {
   return s;
 }
 
-int check_launch(const char* what) {
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(TFT_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
-  return TFT_OK;
-}
-
 int check_chunk_elems(const char* what, uint32_t chunk_elems) {
   if (chunk_elems < TFT_MIN_CHUNK_ELEMS || !is_pow2(chunk_elems))
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: chunk_elems %u is not a power of two >= %u", what,
@@ -495,11 +587,17 @@ int check_chunk_elems(const char* what, uint32_t chunk_elems) {
   return TFT_OK;
 }
 
-// One workgroup per slab and slab indices are 32-bit; the smallest slab any
+// One workgroup per slab and slab indices are 32-bit, including the padding of the
+// grid (up to one row of kMaxGridX and one group of 8 runs); the smallest slab any
 // kernel uses is 1024 elements (4096 bytes for the copy kernel).
-uint32_t max_chunks(uint32_t chunk_elems) { return 0xffffffffu / (chunk_elems / 1024u); }
+constexpr uint32_t kMaxSlabs = 0xffffffffu - 2u * kMaxGridX;
+uint32_t max_chunks(uint32_t chunk_elems) { return kMaxSlabs / (chunk_elems / 1024u); }
 
-dim3 grid_for(uint64_t slabs) {
+// Grid for `slabs` workgroups, padded to whole groups of 8 runs (slab_index is a
+// permutation of [0, padded)); kMaxGridX is a multiple of every group size.
+dim3 grid_for(uint64_t slabs, uint32_t run_log2) {
+  const uint64_t group = 8ull << run_log2;
+  slabs = (slabs + group - 1) / group * group;
   const uint32_t x = (uint32_t)(slabs < kMaxGridX ? slabs : kMaxGridX);
   const uint32_t y = (uint32_t)((slabs + x - 1) / x);
   return dim3(x, y, 1);
@@ -533,46 +631,81 @@ int check_reduce(const char* what, uint32_t n_replicas, uint32_t mask, uint32_t 
   return TFT_OK;
 }
 
+int check_dtype(const char* what, int dtype) {
+  if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
+  return TFT_OK;
+}
+
+uint32_t popcount(uint32_t x) { return (uint32_t)__builtin_popcount(x); }
+
+// The launch itself; the return code of hipLaunchKernel is this launch's own
+// (the sticky "last error" may belong to somebody else's earlier call).
+template <class Args, class Op>
+int launch_kernel(const char* what, const void* kernel, dim3 grid, uint32_t lds, hipStream_t stream,
+                  Args& a, Op& op) {
+  void* params[] = {&a, &op};
+  const hipError_t e = hipLaunchKernel(kernel, grid, dim3(kThreads), params, lds, stream);
+  if (e != hipSuccess) return fail(TFT_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return TFT_OK;
+}
+
 // slab_elems always divides chunk_elems: both are powers of two and
 // chunk_elems >= TFT_MIN_CHUNK_ELEMS >= the largest slab (256 lanes * 8 bf16 * 4;
 // 256 lanes * 16 bytes * 4 for the byte copy, whose minimum is checked there).
-TableArgs table_args(const tft_mt_table* t, uint32_t slab_elems, dim3* grid) {
+TableArgs table_args(const tft_mt_table* t, uint32_t slab_elems, const Shape& shape, dim3* grid) {
   const uint32_t shift = log2u(t->chunk_elems / slab_elems);
-  *grid = grid_for((uint64_t)t->total_chunks << shift);
+  *grid = grid_for((uint64_t)t->total_chunks << shift, shape.run_log2);
   return TableArgs{static_cast<void* const*>(t->ptrs), t->numel, t->chunk_start, t->chunk_tensor,
-                   t->n_tensors, t->chunk_elems, shift, t->total_chunks};
+                   t->n_tensors, t->chunk_elems, shift, t->total_chunks, shape.run_log2};
 }
 
 template <class E, class Op, int U, bool NT>
-void launch_table(const tft_mt_table* t, const Op& op, hipStream_t stream) {
+int launch_table(const char* what, const tft_mt_table* t, const Op& op, const Shape& shape,
+                 hipStream_t stream) {
   dim3 grid;
-  const TableArgs a = table_args(t, kThreads * E::kVec * U, &grid);
-  hipLaunchKernelGGL((mt_stream_kernel<E, Op, TableLocator<Op::NCOL>, U, NT>), grid,
-                     dim3(kThreads), 0, stream, a, op);
+  TableArgs a = table_args(t, kThreads * E::kVec * U, shape, &grid);
+  Op o = op;
+  return launch_kernel(what, reinterpret_cast<const void*>(
+                                 &mt_stream_kernel<E, Op, TableLocator<Op::NCOL>, U, NT>),
+                       grid, shape.lds_bytes, stream, a, o);
 }
 
 template <class E, class Op, int U, bool NT>
-void launch_flat(const FlatArgs& a, const Op& op, hipStream_t stream) {
+int launch_flat(const char* what, const FlatArgs& args, const Op& op, const Shape& shape,
+                hipStream_t stream) {
   const uint64_t slab = (uint64_t)kThreads * E::kVec * U;
-  const dim3 grid = grid_for((a.numel + slab - 1) / slab);
-  hipLaunchKernelGGL((mt_stream_kernel<E, Op, FlatLocator<Op::NCOL>, U, NT>), grid,
-                     dim3(kThreads), 0, stream, a, op);
+  FlatArgs a = args;
+  a.run_log2 = shape.run_log2;
+  // one extra slab: a misaligned buffer's body is shifted by up to 15 bytes
+  const dim3 grid = grid_for((a.numel + slab - 1) / slab + 1, shape.run_log2);
+  Op o = op;
+  return launch_kernel(what, reinterpret_cast<const void*>(
+                                 &mt_stream_kernel<E, Op, FlatLocator<Op::NCOL>, U, NT>),
+                       grid, shape.lds_bytes, stream, a, o);
 }
 
-// Expands to the launch of LAUNCHER<E, Op, U, NT>(ARGS, op, stream) for the
-// thread's launch variant.
-#define TFT_DISPATCH_VARIANT(LAUNCHER, E, OP, ARGS, op, stream, DEFAULT_U)         \
-  do {                                                                             \
-    const Variant v_ = decode_variant(DEFAULT_U);                                  \
-    if (v_.nt) {                                                                   \
-      if (v_.unroll == 4) LAUNCHER<E, OP, 4, true>(ARGS, op, stream);              \
-      else if (v_.unroll == 2) LAUNCHER<E, OP, 2, true>(ARGS, op, stream);         \
-      else LAUNCHER<E, OP, 1, true>(ARGS, op, stream);                             \
-    } else {                                                                       \
-      if (v_.unroll == 4) LAUNCHER<E, OP, 4, false>(ARGS, op, stream);             \
-      else if (v_.unroll == 2) LAUNCHER<E, OP, 2, false>(ARGS, op, stream);        \
-      else LAUNCHER<E, OP, 1, false>(ARGS, op, stream);                            \
-    }                                                                              \
+// rc = LAUNCHER<E, OP, U, NT>(what, ARGS, op, shape, stream) for the shape's unroll
+// (plain instead of non-temporal accesses exist in tuning builds only).
+#ifdef TFT_TUNING
+#define TFT_DISPATCH_NT(LAUNCHER, E, OP, UU, what, ARGS, op, shape, stream)       \
+  ((shape).nt ? LAUNCHER<E, OP, UU, true>(what, ARGS, op, shape, stream)          \
+              : LAUNCHER<E, OP, UU, false>(what, ARGS, op, shape, stream))
+#else
+#define TFT_DISPATCH_NT(LAUNCHER, E, OP, UU, what, ARGS, op, shape, stream) \
+  LAUNCHER<E, OP, UU, true>(what, ARGS, op, shape, stream)
+#endif
+#define TFT_DISPATCH_U(rc, LAUNCHER, E, OP, what, ARGS, op, shape, stream)                          \
+  do {                                                                                              \
+    if ((shape).unroll == 4) rc = TFT_DISPATCH_NT(LAUNCHER, E, OP, 4, what, ARGS, op, shape, stream);      \
+    else if ((shape).unroll == 2) rc = TFT_DISPATCH_NT(LAUNCHER, E, OP, 2, what, ARGS, op, shape, stream); \
+    else rc = TFT_DISPATCH_NT(LAUNCHER, E, OP, 1, what, ARGS, op, shape, stream);                          \
+  } while (0)
+#define TFT_DISPATCH_DTYPE(rc, LAUNCHER, OP, dtype, what, ARGS, op, shape, stream)            \
+  do {                                                                                        \
+    if ((dtype) == TFT_F32) TFT_DISPATCH_U(rc, LAUNCHER, F32, OP, what, ARGS, op, shape, stream);        \
+    else if ((dtype) == TFT_BF16) TFT_DISPATCH_U(rc, LAUNCHER, BF16, OP, what, ARGS, op, shape, stream); \
+    else TFT_DISPATCH_U(rc, LAUNCHER, F16, OP, what, ARGS, op, shape, stream);                           \
   } while (0)
 
 // Expands `CALL(N)` for the run-time replica count.
@@ -609,6 +742,32 @@ int check_sgd(const char* what, const tft_sgd_params* s) {
   return TFT_OK;
 }
 
+uint64_t esize_of(int dtype) { return dtype == TFT_F32 ? 4 : 2; }
+
+// elements a table covers, rounded up to whole chunks (the host does not read the
+// device-resident sizes); only used to choose the launch shape
+uint64_t table_elems(const tft_mt_table* t) { return (uint64_t)t->total_chunks * t->chunk_elems; }
+
+int diloco_outer(const char* what, const tft_mt_table* table, uint32_t n_replicas,
+                 uint32_t participate_mask, uint32_t num_participants, int dtype,
+                 const tft_sgd_params* sgd, void* stream) {
+  const SgdCoef k = make_coef(sgd);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint32_t streams = popcount(participate_mask) + 2 + (k.momentum != 0.0f ? (k.first_step ? 1 : 2) : 0);
+  const Shape shape = pick_shape(kFamDiloco, table_elems(table) * esize_of(dtype) * streams);
+  int rc = TFT_OK;
+#define TFT_CALL(N)                                                                     \
+  do {                                                                                  \
+    typedef DilocoFusedOp<N> Op;                                                        \
+    const Op op{participate_mask, (float)num_participants, k};                          \
+    TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);         \
+  } while (0)
+  TFT_FOR_NREP(n_replicas, TFT_CALL)
+#undef TFT_CALL
+  return rc;
+}
+
+
 }  // namespace
 
 extern "C" {
@@ -617,7 +776,9 @@ int tft_abi_version(void) { return TFT_ABI_VERSION; }
 
 const char* tft_last_error(void) { return g_err; }
 
+#ifdef TFT_TUNING
 void tft_set_launch_variant(uint32_t variant) { g_variant = variant; }
+#endif
 
 uint32_t tft_default_chunk_elems(int dtype) {
   if (dtype < 0) return 256u * 1024u;  // bytes per copy chunk
@@ -649,8 +810,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
                    int dtype, void* stream) {
   static const char* what = "tft_reduce_avg";
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
-    return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
+  if (int rc = check_dtype(what, dtype)) return rc;
   if (numel == 0) return TFT_OK;
   if (!out) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: out is NULL", what);
   if (n_replicas && !replicas) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: replicas is NULL", what);
@@ -664,20 +824,18 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
   }
   a.numel = numel;
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define TFT_CALL(N)                                                            \
-  do {                                                                         \
-    typedef ReduceAvgOp<1, N> Op;                                              \
-    const Op op{participate_mask, (float)num_participants};                    \
-    if (dtype == TFT_F32)                                                      \
-      TFT_DISPATCH_VARIANT(launch_flat, F32, Op, a, op, s, 4);                 \
-    else if (dtype == TFT_BF16)                                                \
-      TFT_DISPATCH_VARIANT(launch_flat, BF16, Op, a, op, s, 4);                \
-    else                                                                       \
-      TFT_DISPATCH_VARIANT(launch_flat, F16, Op, a, op, s, 4);                 \
+  const Shape shape =
+      pick_shape(kFamReduce, numel * esize_of(dtype) * (popcount(participate_mask) + 1));
+  int rc = TFT_OK;
+#define TFT_CALL(N)                                                             \
+  do {                                                                          \
+    typedef ReduceAvgOp<1, N> Op;                                               \
+    const Op op{participate_mask, (float)num_participants};                     \
+    TFT_DISPATCH_DTYPE(rc, launch_flat, Op, dtype, what, a, op, shape, s);      \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
-  return check_launch(what);
+  return rc;
 }
 
 int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_replicas,
@@ -687,20 +845,17 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
   if (n_outs != 1 && n_outs != 2)
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: n_outs must be 1 or 2, got %u", what, n_outs);
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
-    return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
+  if (int rc = check_dtype(what, dtype)) return rc;
   if (int rc = check_table(what, table, n_outs + n_replicas)) return rc < 0 ? rc : TFT_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define TFT_CALL2(O, N)                                                        \
-  do {                                                                         \
-    typedef ReduceAvgOp<O, N> Op;                                              \
-    const Op op{participate_mask, (float)num_participants};                    \
-    if (dtype == TFT_F32)                                                      \
-      TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 4);            \
-    else if (dtype == TFT_BF16)                                                \
-      TFT_DISPATCH_VARIANT(launch_table, BF16, Op, table, op, s, 4);           \
-    else                                                                       \
-      TFT_DISPATCH_VARIANT(launch_table, F16, Op, table, op, s, 4);            \
+  const Shape shape = pick_shape(
+      kFamReduce, table_elems(table) * esize_of(dtype) * (popcount(participate_mask) + n_outs));
+  int rc = TFT_OK;
+#define TFT_CALL2(O, N)                                                               \
+  do {                                                                                \
+    typedef ReduceAvgOp<O, N> Op;                                                     \
+    const Op op{participate_mask, (float)num_participants};                           \
+    TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);       \
   } while (0)
 #define TFT_CALL_O1(N) TFT_CALL2(1, N)
 #define TFT_CALL_O2(N) TFT_CALL2(2, N)
@@ -712,55 +867,55 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
 #undef TFT_CALL_O1
 #undef TFT_CALL_O2
 #undef TFT_CALL2
-  return check_launch(what);
+  return rc;
 }
 
-int tft_mt_diloco_outer_f32(const tft_mt_table* table, uint32_t n_replicas,
-                            uint32_t participate_mask, uint32_t num_participants,
-                            const tft_sgd_params* sgd, void* stream) {
-  static const char* what = "tft_mt_diloco_outer_f32";
+int tft_mt_diloco_outer(const tft_mt_table* table, uint32_t n_replicas, uint32_t participate_mask,
+                        uint32_t num_participants, int dtype, const tft_sgd_params* sgd,
+                        void* stream) {
+  static const char* what = "tft_mt_diloco_outer";
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (int rc = check_dtype(what, dtype)) return rc;
   if (int rc = check_sgd(what, sgd)) return rc;
   if (int rc = check_table(what, table, 3 + n_replicas)) return rc < 0 ? rc : TFT_OK;
-  const SgdCoef k = make_coef(sgd);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-#define TFT_CALL(N)                                                            \
-  do {                                                                         \
-    typedef DilocoFusedOp<N> Op;                                               \
-    const Op op{participate_mask, (float)num_participants, k};                 \
-    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 2);              \
-  } while (0)
-  TFT_FOR_NREP(n_replicas, TFT_CALL)
-#undef TFT_CALL
-  return check_launch(what);
+  return diloco_outer(what, table, n_replicas, participate_mask, num_participants, dtype, sgd, stream);
 }
 
-int tft_mt_pseudograd_avg_f32(const tft_mt_table* table, uint32_t n_replicas,
-                              uint32_t participate_mask, uint32_t num_participants,
-                              int restore_p, void* stream) {
-  static const char* what = "tft_mt_pseudograd_avg_f32";
+int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
+                          uint32_t participate_mask, uint32_t num_participants, int dtype,
+                          int restore_p, void* stream) {
+  static const char* what = "tft_mt_pseudograd_avg";
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (int rc = check_dtype(what, dtype)) return rc;
   if (int rc = check_table(what, table, 3 + n_replicas)) return rc < 0 ? rc : TFT_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const Shape shape = pick_shape(
+      kFamPseudograd,
+      table_elems(table) * esize_of(dtype) * (popcount(participate_mask) + 2 + (restore_p ? 1 : 0)));
+  int rc = TFT_OK;
 #define TFT_CALL(N)                                                                   \
   do {                                                                                \
     typedef PseudogradOp<N> Op;                                                       \
     const Op op{participate_mask, (float)num_participants, restore_p ? 1u : 0u};      \
-    TFT_DISPATCH_VARIANT(launch_table, F32, Op, table, op, s, 2);                     \
+    TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);       \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
-  return check_launch(what);
+  return rc;
 }
 
-int tft_mt_outer_sgd_f32(const tft_mt_table* table, const tft_sgd_params* sgd, void* stream) {
-  static const char* what = "tft_mt_outer_sgd_f32";
+int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd,
+                     void* stream) {
+  static const char* what = "tft_mt_outer_sgd";
+  if (int rc = check_dtype(what, dtype)) return rc;
   if (int rc = check_sgd(what, sgd)) return rc;
   if (int rc = check_table(what, table, 4)) return rc < 0 ? rc : TFT_OK;
   const OuterSgdOp op{make_coef(sgd)};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  TFT_DISPATCH_VARIANT(launch_table, F32, OuterSgdOp, table, op, s, 2);
-  return check_launch(what);
+  const Shape shape = pick_shape(kFamOuterSgd, table_elems(table) * esize_of(dtype) * 6);
+  int rc = TFT_OK;
+  TFT_DISPATCH_DTYPE(rc, launch_table, OuterSgdOp, dtype, what, table, op, shape, s);
+  return rc;
 }
 
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
@@ -769,25 +924,31 @@ int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
   if (table->chunk_elems < kThreads * 16 * 4)
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: chunk_elems %u bytes is below %d", what,
                 table->chunk_elems, kThreads * 16 * 4);
-  const Variant v = decode_variant(1);
+  const Shape shape = pick_shape(kFamCopy, table_elems(table) * 2);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid;
-#define TFT_COPY(UU, NTT)                                                        \
-  do {                                                                           \
-    const TableArgs a = table_args(table, kThreads * 16 * UU, &grid);            \
-    hipLaunchKernelGGL((mt_copy_kernel<UU, NTT>), grid, dim3(kThreads), 0, s, a); \
+  int rc = TFT_OK;
+#define TFT_COPY(UU, NTT)                                                                      \
+  do {                                                                                         \
+    TableArgs a = table_args(table, kThreads * 16 * UU, shape, &grid);                         \
+    void* params[] = {&a};                                                                     \
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(&mt_copy_kernel<UU, NTT>), \
+                                         grid, dim3(kThreads), params, shape.lds_bytes, s);    \
+    if (e != hipSuccess) rc = fail(TFT_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e)); \
   } while (0)
-  if (v.nt) {
-    if (v.unroll == 4) TFT_COPY(4, true);
-    else if (v.unroll == 2) TFT_COPY(2, true);
-    else TFT_COPY(1, true);
-  } else {
-    if (v.unroll == 4) TFT_COPY(4, false);
-    else if (v.unroll == 2) TFT_COPY(2, false);
+#ifdef TFT_TUNING
+  if (!shape.nt) {
+    if (shape.unroll == 4) TFT_COPY(4, false);
+    else if (shape.unroll == 2) TFT_COPY(2, false);
     else TFT_COPY(1, false);
+    return rc;
   }
+#endif
+  if (shape.unroll == 4) TFT_COPY(4, true);
+  else if (shape.unroll == 2) TFT_COPY(2, true);
+  else TFT_COPY(1, true);
 #undef TFT_COPY
-  return check_launch(what);
+  return rc;
 }
 
 }  // extern "C"

@@ -43,6 +43,9 @@ from .multi_tensor import TensorTable
 logger: logging.Logger = logging.getLogger(__name__)
 
 
+_KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
 def _is_native_manager(manager: object) -> bool:
     # a create_autospec(Manager) double passes isinstance() but is not a subclass instance
     return issubclass(type(manager), Manager)
@@ -168,6 +171,14 @@ class LocalSGD:
                 self._backup_parameters[name] = t
         if named and any(p.is_cuda for _, p in named):
             _native.lib()  # GPU parameters need the kernels: fail now, loudly, if they are missing
+            # a dtype the kernels do not have is a configuration error: say so here, once,
+            # instead of latching it as a failed all-reduce on every sync
+            bad = sorted({str(p.dtype) for _, p in named if p.is_cuda and p.dtype not in _KERNEL_DTYPES})
+            if bad:
+                raise TypeError(
+                    f"{type(self).__name__}: GPU parameters of {', '.join(bad)}; the replica-sync "
+                    "kernels take float32, bfloat16 and float16"
+                )
         # the first sync needs a valid backup
         self._save_parameters()
 
@@ -281,14 +292,7 @@ class LocalSGD:
         _, params, backups = self._named()
         if self._fused(params, backups):
             if self._manager.reduction_fails_only_at_launch():
-                # a local reduction cannot fail once launched: decide first, then average
-                # and refresh the backup in the same launch
-                if self._manager.should_commit():
-                    self._manager.allreduce_tensors(params, also_write=backups).wait()
-                    if self._manager.errored() is not None:
-                        self._restore_parameters()
-                else:
-                    self._restore_parameters()
+                self._average_single_launch(params, backups)
                 return
             self._manager.allreduce_tensors(params).wait()
         elif _is_native_manager(self._manager) and self._on_device(params, backups):
@@ -297,6 +301,41 @@ class LocalSGD:
             self._average()
         if self._manager.should_commit():
             self._save_parameters()
+        else:
+            self._restore_parameters()
+
+    def _average_single_launch(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> None:
+        """A local reduction cannot fail once launched, so the commit decision is taken
+        first and the sync is ONE launch: the average written to the parameters and the
+        backup together, or (no commit) a plain restore.  Everything that can fail for a
+        reason other than the launch itself (the quorum, finding the peers' buffers,
+        building and validating the tensor table) happens before the vote and is latched
+        like a failed all-reduce; a launch that fails after the vote raises, because the
+        group has already counted the step as committed."""
+        manager = self._manager
+        manager.wait_quorum()  # should_commit reads the quorum's results (async quorum)
+        launches = []
+        if manager.errored() is None:
+            try:
+                replicas, mask = manager.replica_columns(params)
+                for idx in ops.dtype_groups(params):
+                    outs = [[params[i] for i in idx], [backups[i] for i in idx]]
+                    reps = [[rep[i] for i in idx] for rep in replicas]
+                    key = f"average/{params[idx[0]].dtype}"
+                    table = self._tables.get(key)
+                    if table is None or not table.matches([*outs, *reps]):
+                        table = ops.reduce_avg_table(outs, reps)
+                    launches.append((key, outs, reps, mask, table))
+            except Exception as e:  # same latch as Manager.allreduce
+                logger.exception("got exception preparing the fused sync -- skipping: %s", e)
+                manager.report_error(e)
+                launches = []
+        if manager.should_commit():
+            assert launches, "a replica that failed to prepare cannot have voted to commit"
+            for key, outs, reps, mask, table in launches:
+                self._tables[key] = ops.mt_reduce_avg(
+                    outs, reps, mask, manager.num_participants(), table=table
+                )
         else:
             self._restore_parameters()
 
@@ -321,8 +360,10 @@ class LocalSGD:
 def _fusable_sgd(
     optimizer: optim.Optimizer, params: Sequence[torch.Tensor]
 ) -> Optional[List[Tuple[List[int], ops.OuterSGD, bool]]]:
-    """If ``optimizer`` is a plain ``torch.optim.SGD`` over exactly ``params``, returns per
-    parameter group (indices into ``params``, hyper-parameters, first_step); else None."""
+    """If ``optimizer`` is a plain ``torch.optim.SGD`` over exactly ``params``, returns one
+    entry per (parameter group, dtype): (indices into ``params``, hyper-parameters,
+    first_step); else None.  fp32, bf16 and fp16 parameters are fused (16-bit storage
+    with fp32 arithmetic); the momentum buffer has the parameter's dtype, as torch's has."""
     if type(optimizer) is not optim.SGD:
         return None
     index = {p.data_ptr(): i for i, p in enumerate(params)}
@@ -334,19 +375,6 @@ def _fusable_sgd(
         lr = group["lr"]
         if isinstance(lr, torch.Tensor):
             return None
-        idx = []
-        have_buf = []
-        for p in group["params"]:
-            i = index.get(p.data_ptr())
-            if i is None or p.dtype != torch.float32:
-                return None
-            idx.append(i)
-            have_buf.append(optimizer.state.get(p, {}).get("momentum_buffer") is not None)
-        if not idx:
-            continue
-        if any(have_buf) != all(have_buf):
-            return None
-        covered += len(idx)
         sgd = ops.OuterSGD(
             lr=float(lr),
             momentum=float(group["momentum"]),
@@ -354,7 +382,22 @@ def _fusable_sgd(
             weight_decay=float(group["weight_decay"]),
             nesterov=bool(group["nesterov"]),
         )
-        plan.append((idx, sgd, not all(have_buf)))
+        by_dtype: Dict[torch.dtype, Tuple[List[int], List[bool]]] = {}
+        for p in group["params"]:
+            i = index.get(p.data_ptr())
+            if i is None or p.dtype not in _KERNEL_DTYPES:
+                return None
+            buf = optimizer.state.get(p, {}).get("momentum_buffer")
+            if buf is not None and (buf.dtype != p.dtype or buf.device != p.device):
+                return None
+            idx, have_buf = by_dtype.setdefault(p.dtype, ([], []))
+            idx.append(i)
+            have_buf.append(buf is not None)
+        for idx, have_buf in by_dtype.values():
+            if any(have_buf) != all(have_buf):
+                return None
+            covered += len(idx)
+            plan.append((idx, sgd, not all(have_buf)))
     if covered != len(params):
         return None
     return plan
@@ -468,10 +511,7 @@ class DiLoCo(LocalSGD):
         elif bucketized:
             # pseudo-gradients written straight into one flat buffer (and the parameters
             # restored) by one launch, then ONE collective for the whole model
-            self._tables["pseudograd"] = ops.mt_pseudograd_avg(
-                grads, params, backups, [params], restore_params=True,
-                table=self._tables.get("pseudograd"),
-            )
+            self._local_pseudograd(grads, params, backups, restore_params=True)
             for p, g in zip(live, grads):
                 p.grad = g
             works = [self._manager.allreduce(flat) for flat in self._flat_like("grads", params)[0].values()]
@@ -479,10 +519,7 @@ class DiLoCo(LocalSGD):
                 work.wait()
         else:
             # pseudo-gradients in one launch, then the Manager contract per parameter
-            self._tables["pseudograd"] = ops.mt_pseudograd_avg(
-                grads, params, backups, [params], restore_params=False,
-                table=self._tables.get("pseudograd"),
-            )
+            self._local_pseudograd(grads, params, backups, restore_params=False)
             for p, g in zip(live, grads):
                 p.grad = g
             self._average_grads()
@@ -491,6 +528,23 @@ class DiLoCo(LocalSGD):
         if self._manager.should_commit():
             self._outer_step(params, backups, grads, plan)
         self._outer_optimizer.zero_grad()
+
+    def _local_pseudograd(
+        self,
+        grads: List[torch.Tensor],
+        params: List[torch.Tensor],
+        backups: List[torch.Tensor],
+        restore_params: bool,
+    ) -> None:
+        """This replica's own pseudo-gradients ``params - backups`` (torchft/local_sgd.py:212-215),
+        one launch per dtype; optionally restores the parameters in the same pass."""
+        for idx in ops.dtype_groups(params):
+            key = f"pseudograd/{params[idx[0]].dtype}"
+            sub = [[col[i] for i in idx] for col in (grads, params, backups)]
+            self._tables[key] = ops.mt_pseudograd_avg(
+                sub[0], sub[1], sub[2], [sub[1]], restore_params=restore_params,
+                table=self._tables.get(key),
+            )
 
     def _sync_single_launch(
         self,
@@ -515,15 +569,23 @@ class DiLoCo(LocalSGD):
                         bufs=bufs,
                         replicas=[[rep[i] for i in idx] for rep in replicas],
                     )
-                    launches.append((f"fused/{gi}", idx, cols, sgd, first, mask))
+                    key = f"fused/{gi}"
+                    # built (and validated) before the vote: after it only the launch is left
+                    table = ops.diloco_outer_table(
+                        cols["params"], cols["backups"], bufs, cols["replicas"],
+                        table=self._tables.get(key),
+                    )
+                    launches.append((key, idx, cols, sgd, first, mask, table))
             except Exception as e:  # same latch as Manager.allreduce
                 logger.exception("got exception preparing the fused sync -- skipping: %s", e)
                 manager.report_error(e)
+                launches = []
         if manager.should_commit():
-            for key, idx, cols, sgd, first, mask in launches:
+            assert launches or not params, "a replica that failed to prepare cannot have voted to commit"
+            for key, idx, cols, sgd, first, mask, table in launches:
                 self._tables[key] = ops.mt_diloco_outer(
                     cols["params"], cols["backups"], cols["bufs"], cols["replicas"], sgd, first,
-                    mask, manager.num_participants(), table=self._tables.get(key),
+                    mask, manager.num_participants(), table=table,
                 )
                 if first and cols["bufs"] is not None:
                     self._attach_momentum(idx, cols["bufs"])

@@ -29,6 +29,7 @@ from __future__ import annotations
 
 import concurrent.futures
 import logging
+import os
 from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass, field
 from datetime import timedelta
@@ -39,7 +40,7 @@ import torch
 from torch.distributed import ReduceOp
 
 from . import ops
-from .checkpointing import CheckpointTransport
+from .checkpointing import CheckpointServer, CheckpointTransport
 from .futures import future_timeout
 from .multi_tensor import TensorTable
 
@@ -151,29 +152,60 @@ def _done_future(value: object) -> torch.futures.Future:
 class Manager(Generic[T]):
     """Fault-tolerant step bookkeeping plus the averaged all-reduce.
 
-    Args mirror the reference constructor (torchft/manager.py:87-108) where they
-    concern this path: ``pg``, ``load_state_dict``, ``state_dict``,
-    ``min_replica_size``, ``use_async_quorum``, ``timeout``, ``quorum_timeout``,
-    ``rank``, ``world_size_mode``, ``checkpoint_transport``.  Rendezvous and
-    server arguments of the reference (store / lighthouse addresses, ports) are
-    replaced by ``quorum_client``.
+    The constructor takes the reference's arguments in the reference's order
+    (torchft/manager.py:87-108), so a call written for torchft binds the same way.
+    What the arguments *do* differs for the control plane, which is not part of
+    this package: ``store_addr`` / ``store_port`` / ``lighthouse_addr`` / ``port`` /
+    ``hostname`` / ``heartbeat_interval`` / ``connect_timeout`` / ``world_size``
+    describe the reference's TCPStore rendezvous and its Rust manager server.
+    Here the quorum comes from ``quorum_client`` (an extra, keyword-only seat for
+    the reference's ``ManagerClient``); a call that names a lighthouse, a store or
+    a server port without giving a ``quorum_client`` is refused with one clear
+    error instead of silently training without fault tolerance.  With neither,
+    the manager runs a static single-group quorum over ``pg.size()`` replicas.
     """
 
     def __init__(
         self,
         pg,
-        load_state_dict: Optional[Callable[[T], None]] = None,
-        state_dict: Optional[Callable[[], T]] = None,
-        min_replica_size: int = 1,
+        load_state_dict: Optional[Callable[[T], None]],
+        state_dict: Optional[Callable[[], T]],
+        min_replica_size: int,
         use_async_quorum: bool = True,
         timeout: timedelta = timedelta(seconds=60),
         quorum_timeout: timedelta = timedelta(seconds=60),
-        rank: int = 0,
+        connect_timeout: timedelta = timedelta(seconds=60),
+        rank: Optional[int] = None,
+        world_size: Optional[int] = None,
         world_size_mode: WorldSizeMode = WorldSizeMode.DYNAMIC,
+        store_addr: Optional[str] = None,
+        store_port: Optional[int] = None,
+        lighthouse_addr: Optional[str] = None,
         replica_id: Optional[str] = None,
+        port: Optional[int] = None,
+        hostname: Optional[str] = None,
+        heartbeat_interval: timedelta = timedelta(milliseconds=100),
         checkpoint_transport: Optional[CheckpointTransport] = None,
+        *,
         quorum_client: Optional[QuorumClient] = None,
     ) -> None:
+        if quorum_client is None:
+            named = {
+                "lighthouse_addr": lighthouse_addr,
+                "store_addr": store_addr,
+                "store_port": store_port,
+                "port": port,
+                "TORCHFT_LIGHTHOUSE (environment)": os.environ.get("TORCHFT_LIGHTHOUSE"),
+            }
+            given = [k for k, v in named.items() if v is not None]
+            if given:
+                raise NotImplementedError(
+                    "control plane not built; pass quorum_client=: this package has no lighthouse / "
+                    "manager server / TCPStore rendezvous, and " + ", ".join(given) + " was given. "
+                    "Seat a client with torchft's ManagerClient interface via "
+                    "quorum_client=ManagerClientAdapter(client)."
+                )
+            quorum_client = StaticQuorum(0, pg.size())
         self._pg = pg
         self._load_state_dict = load_state_dict
         self._user_state_dict = state_dict
@@ -181,11 +213,16 @@ class Manager(Generic[T]):
         self._use_async_quorum = use_async_quorum
         self._timeout = timeout
         self._quorum_timeout = quorum_timeout
-        self._rank = rank
+        self._connect_timeout = connect_timeout
+        self._rank: int = rank if rank is not None else int(os.environ.get("RANK", 0))
         self._world_size_mode = world_size_mode
         self._replica_id = replica_id or ""
-        self._checkpoint_transport = checkpoint_transport
-        self._client: QuorumClient = quorum_client or StaticQuorum(0, pg.size())
+        if checkpoint_transport is None and not isinstance(quorum_client, StaticQuorum):
+            # the reference's default (torchft/manager.py:155-158); a static quorum never
+            # asks anybody to heal, so it gets no server thread
+            checkpoint_transport = CheckpointServer(timeout=timeout)
+        self._checkpoint_transport: Optional[CheckpointTransport] = checkpoint_transport
+        self._client: QuorumClient = quorum_client
 
         self._executor = ThreadPoolExecutor(max_workers=1, thread_name_prefix="async_quorum")
         self._quorum_future: Optional[concurrent.futures.Future] = None
@@ -413,7 +450,10 @@ class Manager(Generic[T]):
 
         Never raises: a failure is latched (``errored()``), the future still
         completes with the (possibly corrupt) tensor and every later call is a no-op
-        until the next ``start_quorum`` (torchft/manager.py:242-303)."""
+        until the next ``start_quorum`` (torchft/manager.py:242-303).  The one exception is
+        a tensor the kernels cannot take at all (CPU, non-contiguous, unsupported dtype):
+        that is a configuration error and raises, instead of blocking every commit."""
+        ops.check_tensor(tensor, "Manager.allreduce")
         if self.errored():
             return _done_future(tensor)
         self.wait_quorum()
@@ -461,12 +501,16 @@ class Manager(Generic[T]):
         self.wait_quorum()
         try:
             replicas, mask = self.replica_columns(tensors)
-            outs = [tensors] + ([list(also_write)] if also_write is not None else [])
-            cols = [*outs, *replicas]
-            key = "allreduce_tensors/%d" % len(outs)
-            self._tables[key] = ops.mt_reduce_avg(
-                outs, replicas, mask, self.num_participants(), table=self._cached_table(key, cols)
-            )
+            for idx in ops.dtype_groups(tensors):
+                outs = [[tensors[i] for i in idx]]
+                if also_write is not None:
+                    outs.append([also_write[i] for i in idx])
+                reps = [[rep[i] for i in idx] for rep in replicas]
+                key = "allreduce_tensors/%d/%s" % (len(outs), tensors[idx[0]].dtype)
+                self._tables[key] = ops.mt_reduce_avg(
+                    outs, reps, mask, self.num_participants(),
+                    table=self._cached_table(key, [*outs, *reps]),
+                )
             return self.wrap_future(_done_future(tensors), tensors)
         except Exception as e:
             logger.exception("%s got exception in all reduce -- skipping remaining: %s", self._tag(), e)
@@ -489,12 +533,13 @@ class Manager(Generic[T]):
         self.wait_quorum()
         try:
             replicas, mask = self.replica_columns(params)
-            cols = [grads, params, backups, *replicas]
-            key = "pseudograd"
-            self._tables[key] = ops.mt_pseudograd_avg(
-                grads, params, backups, replicas, restore_params, mask, self.num_participants(),
-                table=self._cached_table(key, cols),
-            )
+            for idx in ops.dtype_groups(params):
+                cols = [[col[i] for i in idx] for col in (grads, params, backups, *replicas)]
+                key = "pseudograd/%s" % params[idx[0]].dtype
+                self._tables[key] = ops.mt_pseudograd_avg(
+                    cols[0], cols[1], cols[2], cols[3:], restore_params, mask,
+                    self.num_participants(), table=self._cached_table(key, cols),
+                )
             return self.wrap_future(_done_future(grads), grads)
         except Exception as e:
             logger.exception("%s got exception in all reduce -- skipping remaining: %s", self._tag(), e)

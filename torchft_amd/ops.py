@@ -45,6 +45,13 @@ class OuterSGD:
         )
 
 
+def check_tensor(t: torch.Tensor, what: str) -> None:
+    """Raises for a tensor no kernel can take (not on a GPU, not contiguous, or of a dtype
+    other than fp32 / bf16 / fp16): a configuration error, never a transient failure."""
+    require_device_tensor(t, what)
+    dtype_code(t.dtype)
+
+
 def full_mask(n_replicas: int) -> int:
     return (1 << n_replicas) - 1
 
@@ -124,9 +131,19 @@ def mt_reduce_avg(
     return table
 
 
-def _require_f32(table: TensorTable, what: str) -> None:
-    if table.dtype is not torch.float32:
-        raise TypeError(f"{what}: fp32 tensors only, got {table.dtype}")
+def diloco_outer_table(
+    params: Sequence[torch.Tensor],
+    backups: Sequence[torch.Tensor],
+    bufs: Optional[Sequence[torch.Tensor]],
+    replicas: Sequence[Sequence[torch.Tensor]],
+    table: Optional[TensorTable] = None,
+) -> TensorTable:
+    """The tensor table of :func:`mt_diloco_outer` (validates devices, dtypes and sizes;
+    ``table`` is returned as is when it still describes the same tensors)."""
+    cols = [params, backups, bufs if bufs is not None else backups, *replicas]
+    if table is not None and table.matches(cols):
+        return table
+    return TensorTable(cols, what="mt_diloco_outer")
 
 
 def mt_diloco_outer(
@@ -140,19 +157,18 @@ def mt_diloco_outer(
     num_participants: Optional[int] = None,
     table: Optional[TensorTable] = None,
 ) -> TensorTable:
-    """Fused DiLoCo outer step (pseudo-gradient, average, Nesterov SGD, backup refresh)."""
+    """Fused DiLoCo outer step (pseudo-gradient, average, Nesterov SGD, backup refresh);
+    fp32, or bf16 / fp16 storage with fp32 arithmetic and one rounding on store."""
     n = len(replicas)
     mask = full_mask(n) if participate_mask is None else participate_mask
     nump = n if num_participants is None else num_participants
     _check_reduce_args(n, mask, nump)
     if sgd.momentum != 0.0 and bufs is None:
         raise ValueError("momentum != 0 needs momentum buffers")
-    cols = [params, backups, bufs if bufs is not None else backups, *replicas]
-    if table is None or not table.matches(cols):
-        table = TensorTable(cols, what="mt_diloco_outer")
-    _require_f32(table, "mt_diloco_outer")
+    table = diloco_outer_table(params, backups, bufs, replicas, table)
     _launch(
-        table, "tft_mt_diloco_outer_f32", n, mask, nump, ctypes.byref(sgd.to_struct(first_step))
+        table, "tft_mt_diloco_outer", n, mask, nump, table.dtype_code,
+        ctypes.byref(sgd.to_struct(first_step)),
     )
     return table
 
@@ -175,8 +191,9 @@ def mt_pseudograd_avg(
     cols = [grads, params, backups, *replicas]
     if table is None or not table.matches(cols):
         table = TensorTable(cols, what="mt_pseudograd_avg")
-    _require_f32(table, "mt_pseudograd_avg")
-    _launch(table, "tft_mt_pseudograd_avg_f32", n, mask, nump, 1 if restore_params else 0)
+    _launch(
+        table, "tft_mt_pseudograd_avg", n, mask, nump, table.dtype_code, 1 if restore_params else 0
+    )
     return table
 
 
@@ -195,8 +212,9 @@ def mt_outer_sgd(
     cols = [params, backups, bufs if bufs is not None else backups, grads]
     if table is None or not table.matches(cols):
         table = TensorTable(cols, what="mt_outer_sgd")
-    _require_f32(table, "mt_outer_sgd")
-    _launch(table, "tft_mt_outer_sgd_f32", ctypes.byref(sgd.to_struct(first_step)))
+    _launch(
+        table, "tft_mt_outer_sgd", table.dtype_code, ctypes.byref(sgd.to_struct(first_step))
+    )
     return table
 
 
@@ -213,9 +231,14 @@ def mt_copy(
     return table
 
 
-def set_launch_variant(variant: int) -> None:
-    """Benchmark hook; see tft_set_launch_variant in include/torchft_amd.h."""
-    _native.lib().tft_set_launch_variant(variant)
+def dtype_groups(tensors: Sequence[torch.Tensor]) -> List[List[int]]:
+    """Indices of ``tensors`` grouped by dtype, groups in order of first appearance.  One
+    launch covers one dtype (the kernels are instantiated per element type), so a model
+    with bf16 weights and fp32 norms synchronises in two launches."""
+    groups: dict = {}
+    for i, t in enumerate(tensors):
+        groups.setdefault(t.dtype, []).append(i)
+    return list(groups.values())
 
 
 def flat_views(flat: torch.Tensor, like: Sequence[torch.Tensor]) -> List[torch.Tensor]:
