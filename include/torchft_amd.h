@@ -14,7 +14,9 @@
  *   - the library never allocates device memory, never synchronises and keeps
  *     no mutable global state (the error string is thread-local): each call
  *     validates its arguments on the host and enqueues exactly one kernel on the
- *     caller's hipStream_t (passed as void*; NULL is the legacy default stream);
+ *     caller's hipStream_t (passed as void*; NULL is the legacy default stream).
+ *     The one exception is tft_mt_diloco_outer_noalloc, which enqueues a few
+ *     kernels and uses a fixed device array owned by the library;
  *   - re-entrant: may be called concurrently from the training thread, the
  *     autograd thread (DDP comm hook) and the checkpoint thread.
  *
@@ -59,6 +61,7 @@ extern "C" {
 #define TFT_ABI_VERSION 4
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
 #define TFT_MIN_CHUNK_ELEMS 8192u
+#define TFT_NOALLOC_MAX_TENSORS 4096u /* rows of the built-in table of the allocation-free entry */
 
 typedef enum tft_status {
   TFT_OK = 0,
@@ -164,6 +167,30 @@ int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
                           uint32_t participate_mask, uint32_t num_participants, int dtype,
                           int restore_p, void* stream);
 int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd, void* stream);
+
+/*
+ * Allocation-free form of tft_mt_diloco_outer.  It has no counterpart in the
+ * reference: it exists for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc) and
+ * therefore cannot build a tensor table.  The table is built by small kernels,
+ * whose arguments carry its entries, in a fixed 8 MiB array inside the library
+ * (one per GPU), then the same kernel as tft_mt_diloco_outer runs over it; the
+ * call is nothing but kernel launches on `stream` and allocates nothing.
+ *   ptrs   HOST array of (3 + n_replicas) * n_tensors device pointers,
+ *          column-major like a table: ptrs[c * n_tensors + t], columns
+ *          [p, b, buf, replica_0 ..] (buf may be NULL when momentum == 0, a
+ *          replica outside participate_mask may be NULL)
+ *   numel  HOST array of n_tensors element counts, all > 0
+ * Limits: n_tensors <= TFT_NOALLOC_MAX_TENSORS and the table (8 bytes per pointer
+ * and per tensor, 4 bytes per chunk of 65 536 elements) must fit the array, which
+ * holds about 2 million chunks; larger inputs are refused with TFT_ERR_UNSUPPORTED.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one
+ * GPU (different streams or threads) race and must be serialised by the caller.
+ */
+int tft_mt_diloco_outer_noalloc(const void* const* ptrs, const uint64_t* numel, uint32_t n_tensors,
+                                uint32_t n_replicas, uint32_t participate_mask,
+                                uint32_t num_participants, int dtype, const tft_sgd_params* sgd,
+                                void* stream);
 
 /*
  * Byte-exact multi-tensor gather/scatter.  Columns: [dst, src]; numel counts

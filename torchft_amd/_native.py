@@ -22,6 +22,7 @@ ABI_VERSION = 4
 MAX_REPLICAS = 8
 MIN_CHUNK_ELEMS = 8192
 MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
+NOALLOC_MAX_TENSORS = 4096
 
 TFT_F32 = 0
 TFT_BF16 = 1
@@ -72,6 +73,11 @@ SIGNATURES = {
     "tft_mt_diloco_outer": (
         c_int,
         [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_int, POINTER(SgdParams), c_void_p],
+    ),
+    "tft_mt_diloco_outer_noalloc": (
+        c_int,
+        [POINTER(c_void_p), POINTER(c_uint64), c_uint32, c_uint32, c_uint32, c_uint32, c_int,
+         POINTER(SgdParams), c_void_p],
     ),
     "tft_mt_pseudograd_avg": (
         c_int,

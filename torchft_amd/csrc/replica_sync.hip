@@ -23,6 +23,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "torchft_amd.h"
 
 namespace {
@@ -528,6 +530,35 @@ __global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {
 }
 
 // ---------------------------------------------------------------------------
+// Table built on the device, in a fixed array, for the allocation-free entry.
+// ---------------------------------------------------------------------------
+// Callers that cannot allocate device memory (code under graph capture, tight
+// serving loops) cannot build a tensor table either.  For them the table lives in
+// this file-scope array and is written by kernels whose arguments carry the
+// entries, so the whole call is kernel launches on the caller's stream and
+// nothing else.  Each GPU holds its own copy of the array at its own address.
+constexpr size_t kScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr uint32_t kFillWords = 384;  // 64-bit entries carried by one fill launch (3 KiB)
+struct FillArgs {
+  uint64_t v[kFillWords];
+  uint32_t n;
+};
+
+__global__ __launch_bounds__(kThreads) void table_fill_kernel(uint64_t* dst, FillArgs a) {
+  for (uint32_t i = threadIdx.x; i < a.n; i += kThreads) dst[i] = a.v[i];
+}
+
+// chunk_tensor[c] = t for every chunk c of tensor t; one workgroup per tensor
+__global__ __launch_bounds__(kThreads) void table_owner_kernel(const uint32_t* chunk_start,
+                                                               uint32_t* chunk_tensor) {
+  const uint32_t t = blockIdx.x;
+  const uint32_t end = chunk_start[t + 1];
+  for (uint32_t c = chunk_start[t] + threadIdx.x; c < end; c += kThreads) chunk_tensor[c] = t;
+}
+
+// ---------------------------------------------------------------------------
 // Host side: validation, launch shape and dispatch.
 // ---------------------------------------------------------------------------
 
@@ -780,6 +811,48 @@ int diloco_outer(const char* what, const tft_mt_table* table, uint32_t n_replica
 }
 
 
+// Per-device address of `scratch` (the symbol's name is only a host-side handle).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_address(const char* what, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TFT_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: device ordinal %d outside [0, %d)", what, dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(TFT_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", what, dev,
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return TFT_OK;
+}
+
+// Writes `n` 64-bit entries to `dst` (device) with fill launches of kFillWords each.
+int fill_words(const char* what, uint64_t* dst, const uint64_t* src, size_t n, hipStream_t stream) {
+  for (size_t done = 0; done < n; done += kFillWords) {
+    FillArgs a;
+    a.n = (uint32_t)(n - done < kFillWords ? n - done : kFillWords);
+    memcpy(a.v, src + done, a.n * sizeof(uint64_t));
+    uint64_t* d = dst + done;
+    void* params[] = {&d, &a};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(&table_fill_kernel), dim3(1),
+                                         dim3(kThreads), params, 0, stream);
+    if (e != hipSuccess)
+      return fail(TFT_ERR_LAUNCH, "%s: table fill launch failed: %s", what, hipGetErrorString(e));
+  }
+  return TFT_OK;
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
 }  // namespace
 
 extern "C" {
@@ -928,6 +1001,77 @@ int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params*
   int rc = TFT_OK;
   TFT_DISPATCH_DTYPE(rc, launch_table, OuterSgdOp, dtype, what, table, op, shape, s);
   return rc;
+}
+
+int tft_mt_diloco_outer_noalloc(const void* const* ptrs, const uint64_t* numel, uint32_t n_tensors,
+                                uint32_t n_replicas, uint32_t participate_mask,
+                                uint32_t num_participants, int dtype, const tft_sgd_params* sgd,
+                                void* stream) {
+  static const char* what = "tft_mt_diloco_outer_noalloc";
+  if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
+  if (int rc = check_dtype(what, dtype)) return rc;
+  if (int rc = check_sgd(what, sgd)) return rc;
+  if (n_tensors == 0) return TFT_OK;
+  if (!ptrs || !numel) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: ptrs / numel are NULL", what);
+  if (n_tensors > TFT_NOALLOC_MAX_TENSORS)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: %u tensors, at most %u fit the built-in table", what,
+                n_tensors, (unsigned)TFT_NOALLOC_MAX_TENSORS);
+  const uint32_t n_cols = 3 + n_replicas;
+  const bool uses_buf = sgd->momentum != 0.0f;
+  for (uint32_t t = 0; t < n_tensors; ++t) {
+    if (numel[t] == 0)
+      return fail(TFT_ERR_INVALID_ARGUMENT, "%s: tensor %u is empty; drop empty tensors", what, t);
+    for (uint32_t c = 0; c < n_cols; ++c) {
+      const bool used = c < 2 || (c == 2 && uses_buf) || (c >= 3 && ((participate_mask >> (c - 3)) & 1u));
+      if (used && !ptrs[(size_t)c * n_tensors + t])
+        return fail(TFT_ERR_INVALID_ARGUMENT, "%s: column %u of tensor %u is NULL", what, c, t);
+    }
+  }
+  // host-side plan (stack / heap of the host only; nothing on the device is allocated)
+  const uint32_t chunk_elems = tft_default_chunk_elems(dtype);
+  uint32_t chunk_start[TFT_NOALLOC_MAX_TENSORS + 2] = {};
+  const int64_t total = tft_mt_plan(numel, n_tensors, chunk_elems, chunk_start, nullptr);
+  if (total < 0) return (int)total;
+  const size_t off_numel = align_up((size_t)n_cols * n_tensors * 8, 256);
+  const size_t off_start = align_up(off_numel + (size_t)n_tensors * 8, 256);
+  const size_t off_owner = align_up(off_start + (size_t)(n_tensors + 2) * 4, 256);
+  const size_t need = off_owner + (size_t)total * 4;
+  if (need > kScratchBytes)
+    return fail(TFT_ERR_UNSUPPORTED,
+                "%s: the table needs %zu bytes (%lld chunks of %u elements), the built-in array holds %zu",
+                what, need, (long long)total, chunk_elems, kScratchBytes);
+  void* base_v = nullptr;
+  if (int rc = scratch_address(what, &base_v)) return rc;
+  unsigned char* base = static_cast<unsigned char*>(base_v);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (int rc = fill_words(what, reinterpret_cast<uint64_t*>(base),
+                          reinterpret_cast<const uint64_t*>(ptrs), (size_t)n_cols * n_tensors, s))
+    return rc;
+  if (int rc = fill_words(what, reinterpret_cast<uint64_t*>(base + off_numel), numel, n_tensors, s))
+    return rc;
+  // (n_tensors + 1) 32-bit entries travel as 64-bit words; the array has one spare slot
+  if (int rc = fill_words(what, reinterpret_cast<uint64_t*>(base + off_start),
+                          reinterpret_cast<const uint64_t*>(chunk_start), (n_tensors + 2) / 2, s))
+    return rc;
+  {
+    const uint32_t* cs = reinterpret_cast<const uint32_t*>(base + off_start);
+    uint32_t* owner = reinterpret_cast<uint32_t*>(base + off_owner);
+    void* params[] = {&cs, &owner};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(&table_owner_kernel),
+                                         dim3(n_tensors), dim3(kThreads), params, 0, s);
+    if (e != hipSuccess)
+      return fail(TFT_ERR_LAUNCH, "%s: table owner launch failed: %s", what, hipGetErrorString(e));
+  }
+  tft_mt_table table;
+  table.ptrs = base;
+  table.numel = reinterpret_cast<const uint64_t*>(base + off_numel);
+  table.chunk_start = reinterpret_cast<const uint32_t*>(base + off_start);
+  table.chunk_tensor = reinterpret_cast<const uint32_t*>(base + off_owner);
+  table.n_tensors = n_tensors;
+  table.n_cols = n_cols;
+  table.chunk_elems = chunk_elems;
+  table.total_chunks = (uint32_t)total;
+  return diloco_outer(what, &table, n_replicas, participate_mask, num_participants, dtype, sgd, stream);
 }
 
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
