@@ -1,0 +1,122 @@
+"""HBM bank-group placement of the library's own buffers (MI355X): mechanics and, above
+all, that it changes nothing but addresses."""
+
+import pytest
+import torch
+from torch import nn, optim
+
+from helpers import assert_bits_equal
+from oracle import replica_sync as O
+from torchft_amd import (
+    DiLoCo,
+    LocalSGD,
+    Manager,
+    ProcessGroupLocalReplicas,
+    StaticQuorum,
+    hbm_placement as H,
+)
+
+pytestmark = pytest.mark.gpu
+
+
+class Wide(nn.Module):
+    """1.25 GiB of fp32 parameters in tensors large enough to probe, plus small ones."""
+
+    def __init__(self) -> None:
+        super().__init__()
+        self.a = nn.Parameter(torch.empty(160 << 20).normal_(0, 0.02))   # 640 MiB
+        self.b = nn.Parameter(torch.empty(128 << 20).normal_(0, 0.02))   # 512 MiB
+        self.c = nn.Parameter(torch.empty(32 << 20).normal_(0, 0.02))    # 128 MiB
+        self.small = nn.Parameter(torch.empty(1000, 7).normal_(0, 0.02))
+        self.one = nn.Parameter(torch.zeros(1))
+
+
+def test_probe_leaves_the_buffer_unchanged(device):
+    g = torch.Generator(device).manual_seed(0)
+    a = torch.randint(0, 256, (64 << 20,), dtype=torch.uint8, device=device, generator=g)
+    a[:4].copy_(torch.tensor([0xFF, 0xFF, 0xBF, 0x7F], dtype=torch.uint8))  # a signalling NaN pattern
+    keep = a.clone()
+    scratch = torch.zeros_like(a)
+    ms = H.probe_ms(a, scratch)
+    assert ms > 0
+    assert torch.equal(a, keep)
+    assert torch.equal(scratch, keep)  # the copy is exact as well
+
+
+def test_allocate_apart_places_copies_outside_the_models_group(device):
+    torch.manual_seed(0)
+    model = Wide().to(device)
+    like = [p.data for p in model.parameters()]
+    copies = H.allocate_apart(like, 2)
+    assert copies is not None, "no bank-group structure found: is this an MI355X?"
+    seen = set()
+    for col in copies:
+        assert len(col) == len(like)
+        for t, ref in zip(col, like):
+            assert t.shape == ref.shape and t.dtype == ref.dtype and t.device == ref.device
+            assert t.is_contiguous() and t.data_ptr() % 256 == 0
+            span = (t.data_ptr(), t.data_ptr() + t.numel() * t.element_size())
+            assert all(span[1] <= lo or span[0] >= hi for lo, hi in seen), "buffers overlap"
+            seen.add(span)
+    # the probe agrees: a large model tensor and its copies do not share a group, the two
+    # copies of one tensor do (they are kept together)
+    big, copy0, copy1 = like[0], copies[0][0], copies[1][0]
+    half = copy0.numel() // 2
+    same = H.probe_ms(copy0[:half], copy0[half:], 256 << 20)  # two halves of one buffer: one group
+    assert H.probe_ms(big, copy0, 256 << 20) < 0.92 * same
+    assert H.probe_ms(big, copy1, 256 << 20) < 0.92 * same
+    assert H.probe_ms(copy0, copy1, 256 << 20) > 0.92 * same
+    assert_bits_equal(big, model.a.data.cpu())  # probing left the parameters alone
+
+
+@pytest.mark.parametrize("kind", ["diloco", "local_sgd"])
+def test_sync_with_placed_buffers_matches_the_checker(device, kind, monkeypatch):
+    """A model large enough for placement to engage: two syncs through the API, results
+    against the checker bit for bit, and the same again with placement switched off."""
+    results = {}
+    for placement in ("1", "0"):
+        monkeypatch.setenv("TORCHFT_AMD_HBM_PLACEMENT", placement)
+        torch.manual_seed(0)
+        model = Wide().to(device)
+        peer = [p.data + 1e-3 for p in model.parameters()]
+        index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+        pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+        manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                          use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+        inner = optim.SGD(model.parameters(), lr=0.1)
+        outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+        ctx = (DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) if kind == "diloco"
+               else LocalSGD(manager, model, inner, sync_every=10 ** 9))
+        placed = ctx._placed_momentum is not None if kind == "diloco" else None
+        if kind == "diloco":
+            assert placed == (placement == "1")
+        backup = [b.cpu() for b in ctx._backup_parameters.values()]
+        bufs = None
+        with ctx:
+            for step in range(2):
+                with torch.no_grad():
+                    for p in model.parameters():
+                        p.add_(1e-3 * (step + 1))
+                reps = [[p.data.cpu() for p in model.parameters()], [t.cpu() for t in peer]]
+                if kind == "diloco":
+                    want = O.diloco_perform_sync(reps, backup, bufs, [True, True], 2, True, lr=0.7,
+                                                 momentum=0.9, nesterov=True)
+                else:
+                    want = O.localsgd_perform_sync(reps, backup, [True, True], 2, True)
+                ctx.sync()
+                torch.cuda.synchronize()
+                for i, p in enumerate(model.parameters()):
+                    assert_bits_equal(p.data, want["params"][i], f"params[{i}] step {step}")
+                for i, b in enumerate(ctx._backup_parameters.values()):
+                    assert_bits_equal(b, want["backup"][i], f"backup[{i}] step {step}")
+                if kind == "diloco":
+                    for i, p in enumerate(model.parameters()):
+                        assert_bits_equal(outer.state[p]["momentum_buffer"], want["momentum"][i])
+                    bufs = want["momentum"]
+                backup = want["backup"]
+        results[placement] = [p.data.cpu() for p in model.parameters()]
+        manager.shutdown(wait=False)
+        del model, peer, ctx, outer, inner
+        torch.cuda.empty_cache()
+    for x, y in zip(results["1"], results["0"]):
+        assert_bits_equal(x, y)

@@ -85,6 +85,7 @@ SIGNATURES = {
     ),
     "tft_mt_outer_sgd": (c_int, [POINTER(MtTable), c_int, POINTER(SgdParams), c_void_p]),
     "tft_mt_copy_bytes": (c_int, [POINTER(MtTable), c_void_p]),
+    "tft_probe_rw_pair": (c_int, [c_void_p, c_void_p, c_uint64, c_void_p]),
 }
 
 

@@ -466,6 +466,21 @@ struct OuterSgdOp {
   }
 };
 
+// columns: [a, scratch]; a is read and written back unchanged, scratch receives a
+// copy (placement probe: one in-place stream next to one write stream).
+// `key` is zero, but only at run time: storing back exactly what was loaded is
+// something the compiler removes, and the probe exists to be timed.
+struct ProbeOp {
+  static constexpr int NCOL = 2;
+  uint32_t key;
+  __device__ inline uint32_t rmask() const { return 1u; }
+  __device__ inline uint32_t wmask() const { return 3u; }
+  __device__ inline void apply(float (&v)[NCOL]) const {
+    v[0] = __uint_as_float(__float_as_uint(v[0]) ^ key);
+    v[1] = v[0];
+  }
+};
+
 // ---------------------------------------------------------------------------
 // Byte copy (gather / scatter).  columns: [dst, src]; numel counts bytes.
 // ---------------------------------------------------------------------------
@@ -1072,6 +1087,22 @@ int tft_mt_diloco_outer_noalloc(const void* const* ptrs, const uint64_t* numel, 
   table.chunk_elems = chunk_elems;
   table.total_chunks = (uint32_t)total;
   return diloco_outer(what, &table, n_replicas, participate_mask, num_participants, dtype, sgd, stream);
+}
+
+int tft_probe_rw_pair(void* a, void* scratch, uint64_t bytes, void* stream) {
+  static const char* what = "tft_probe_rw_pair";
+  if (bytes == 0) return TFT_OK;
+  if (!a || !scratch) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: buffers must not be NULL", what);
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(scratch) | bytes) & 15u)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: buffers and size must be multiples of 16 bytes", what);
+  if (bytes > (1ull << 40)) return fail(TFT_ERR_UNSUPPORTED, "%s: size too large", what);
+  FlatArgs args{};
+  args.ptrs[0] = a;
+  args.ptrs[1] = scratch;
+  args.numel = bytes / 4;
+  const Shape shape{2, true, 0, 0};
+  const ProbeOp op{0u};
+  return launch_flat<F32, ProbeOp, 2, true>(what, args, op, shape, static_cast<hipStream_t>(stream));
 }
 
 int tft_mt_copy_bytes(const tft_mt_table* table, void* stream) {
