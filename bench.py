@@ -60,9 +60,11 @@ def parse_args() -> argparse.Namespace:
                          "process that has just exited is handed out in a worse physical layout for a "
                          "few seconds (2-5 %% lower bandwidth for the whole run); 0 disables")
     ap.add_argument("--layout", default="",
-                    help="comma list for the DiLoCo workloads: alias_p (the live parameters are replica 0, "
+                    help="comma list: alias_p (DiLoCo workloads: the live parameters are replica 0, "
                          "updated in place), flat_backup / flat_momentum (backup / momentum tensors are "
-                         "views of one flat allocation, back to back without padding)")
+                         "views of one flat allocation, back to back without padding), no_placement "
+                         "(the library allocates backup / momentum / pseudo-gradients without looking "
+                         "at HBM bank groups)")
     ap.add_argument("--arena", action="store_true",
                     help="carve all tensors of the DiLoCo workload out of one device allocation "
                          "instead of allocating each separately (makes no measurable difference)")
@@ -228,7 +230,7 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
                 bufs = views
             del src
             torch.cuda.empty_cache()
-        else:
+        elif item != "no_placement":
             raise SystemExit(f"unknown --layout item {item!r}")
     sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
     table = TensorTable([params, wl.backup, bufs, *wl.replicas], what="bench")
@@ -348,10 +350,18 @@ def bench_diloco_two_phase(args) -> Dict[str, object]:
 
     dev = torch.device("cuda", 0)
     shapes, n_rep = workloads.llama3_8b_shapes(), 2
+    from torchft_amd import hbm_placement
+
     wl = workloads.make_diloco_workload(shapes, n_rep, dev)
     params = wl.replicas[0]  # live parameters are replica 0
-    bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
-    grads = [torch.empty_like(t) for t in wl.backup]
+    # backup, momentum and pseudo-gradients are the library's: allocated the way DiLoCo does
+    backup, bufs = hbm_placement.model_copies(params, 2)
+    grads = hbm_placement.model_copies(params, 1)[0]
+    ops.mt_copy(backup, wl.backup)
+    ops.mt_copy(bufs, workloads.normal_tensors(shapes, 1e-3, 4000, dev))
+    torch.cuda.synchronize()
+    wl.backup = backup
+    torch.cuda.empty_cache()
     sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
     t1 = ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, True)
     t2 = ops.mt_outer_sgd(params, wl.backup, bufs, grads, sgd, False)
@@ -391,8 +401,17 @@ def bench_localsgd(args) -> Dict[str, object]:
     from torchft_amd import ops, workloads
 
     dev = torch.device("cuda", 0)
+    from torchft_amd import hbm_placement
+
     shapes, n_rep = workloads.llama3_8b_shapes(), 2
     wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+    # the backup is the library's: allocated the way LocalSGD does (outside the HBM bank
+    # group of the parameters it shadows)
+    backup = hbm_placement.model_copies(wl.replicas[0], 1)[0]
+    ops.mt_copy(backup, wl.backup)
+    torch.cuda.synchronize()
+    wl.backup = backup
+    torch.cuda.empty_cache()
     table = ops.reduce_avg_table([wl.replicas[0], wl.backup], wl.replicas)
 
     def step() -> None:
@@ -594,6 +613,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
+    if "no_placement" in args.layout.split(","):
+        os.environ["TORCHFT_AMD_HBM_PLACEMENT"] = "0"
     if args.settle_seconds > 0:
         time.sleep(args.settle_seconds)  # before anything is allocated on the device
     torch.cuda.set_device(0)

@@ -588,28 +588,27 @@ struct Shape {
 
 enum Family { kFamReduce, kFamDiloco, kFamPseudograd, kFamOuterSgd, kFamCopy };
 
-// Tuned on MI355X.  `traffic` is the launch's algorithmic bytes: launches that
-// move less than a few GB finish in under a millisecond and are dominated by the
-// ramp and tail of the in-flight window, which a residency cap of two workgroups
-// per CU and short per-XCD runs shorten; large launches want the widest window.
+// Tuned on MI355X with interleaved sweeps over (slab size, per-XCD run, residency cap) on
+// the Llama-3-8B and GPT-2-small workloads.  `traffic` is the launch's algorithmic bytes.
+// Launches that move less than a few GB finish in under a millisecond and are dominated by
+// the ramp and tail of the in-flight window: short runs and 5 resident workgroups per CU
+// (32 KiB of unused LDS each) are worth 5-10 % there.  Large launches still gain 1-5 % from
+// runs of 128-256 slabs with 2-3 resident workgroups per CU; the plain copy is best left
+// alone.
 Shape pick_shape(Family fam, uint64_t traffic) {
-  Shape s{2, true, 0, 0};
   const bool small = traffic < (16ull << 30);
-  switch (fam) {
-    case kFamReduce: s.unroll = small ? 2 : 1; break;
-    case kFamDiloco: s.unroll = small ? 1 : 2; break;
-    case kFamPseudograd: s.unroll = small ? 2 : 1; break;
-    case kFamOuterSgd: s.unroll = small ? 2 : 1; break;
-    case kFamCopy: s.unroll = 1; break;
-  }
-  if (small && fam != kFamCopy) {
+  if (fam == kFamCopy) return Shape{1, true, 0, 0};
+  Shape s{2, true, 0, 0};
+  if (small) {
+    s.unroll = fam == kFamDiloco ? 1 : 2;
     s.run_log2 = fam == kFamDiloco ? 7 : 6;
     s.lds_bytes = 32u << 10;
-  } else if (fam == kFamDiloco) {
-    // large fused step: per-XCD runs of 256 slabs with two resident workgroups per CU
-    // measured 1 % faster than the plain order (34.9 against 35.3 ms on Llama-3-8B)
+  } else if (fam == kFamDiloco || fam == kFamOuterSgd) {
     s.run_log2 = 8;
     s.lds_bytes = 64u << 10;
+  } else {
+    s.run_log2 = 7;
+    s.lds_bytes = 48u << 10;
   }
 #ifdef TFT_TUNING
   // bits 0-3 unroll (1, 2, 4), bit 4 plain accesses, bits 8-11 run_log2 + 1,

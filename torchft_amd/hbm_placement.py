@@ -303,3 +303,12 @@ def allocate_apart(
         len(like), n_copies, n_groups, misplaced,
     )
     return copies
+
+
+def model_copies(like: Sequence[torch.Tensor], n_copies: int) -> List[List[torch.Tensor]]:
+    """``n_copies`` sets of uninitialised tensors shaped like ``like``: placed by bank group
+    where that applies (:func:`allocate_apart`), otherwise one plain allocation per tensor."""
+    placed = allocate_apart(like, n_copies) if n_copies in (1, 2) else None
+    if placed is not None:
+        return placed
+    return [[torch.empty_like(t) for t in like] for _ in range(n_copies)]

@@ -456,7 +456,9 @@ class DiLoCo(LocalSGD):
             g.shape != p.shape or g.device != p.device or g.dtype != p.dtype
             for g, p in zip(self._grads, params)
         ):
-            self._grads = [torch.empty_like(p) for p in params]
+            # written next to the parameters by the pseudo-gradient launch: keep them out of
+            # the parameters' HBM bank group, like the backup
+            self._grads = hbm_placement.model_copies(params, 1)[0]
         return self._grads
 
     def _momentum_buffers(self, idx: Sequence[int], first: bool) -> List[torch.Tensor]:
