@@ -549,6 +549,69 @@ def test_wire_round_trip_through_pinned_host(device):
         state_pack.read_packed(io.BytesIO(data[:len(data) // 2]), device)
 
 
+@pytest.mark.parametrize("chunk_bytes", [4096, 1 << 20, 64 << 20])
+def test_streamed_payload_equals_the_one_shot_pack(device, chunk_bytes):
+    """stream_packed never holds the payload as a whole (three ring slots of chunk_bytes):
+    what it writes must equal the layout of the one-launch pack at every tensor's bytes, for
+    whole payloads and for byte ranges whose concatenation is the payload."""
+    state = _training_state(device)
+    plan = state_pack.plan_pack(state)
+    offsets = [e.offset for e in plan.entries]
+    image = O.gather_bytes(plan.tensors, offsets, plan.total_bytes)
+
+    def payload_of(lo, hi):
+        buf = io.BytesIO()
+        state_pack.stream_packed(plan, buf, lo, hi, chunk_bytes=chunk_bytes)
+        data = buf.getvalue()
+        assert data[:8] == state_pack.MAGIC
+        hlen = int.from_bytes(data[8:16], "little")
+        assert data[16:16 + hlen] == plan.header()
+        return data[16 + hlen:]
+
+    whole = payload_of(0, plan.total_bytes)
+    assert len(whole) == plan.total_bytes
+    for e in plan.entries:
+        assert whole[e.offset:e.offset + e.nbytes] == bytes(image[e.offset:e.offset + e.nbytes])
+    if chunk_bytes >= 1 << 20:
+        parts = [payload_of(*state_pack.split_range(plan.total_bytes, k, 3)) for k in range(3)]
+        joined = b"".join(parts)
+        assert len(joined) == plan.total_bytes
+        for e in plan.entries:
+            assert joined[e.offset:e.offset + e.nbytes] == whole[e.offset:e.offset + e.nbytes]
+    # and the receiving side rebuilds the checker's state from it
+    buf = io.BytesIO()
+    state_pack.stream_packed(plan, buf, chunk_bytes=chunk_bytes)
+    buf.seek(0)
+    header, staging = state_pack.read_packed(buf, device, chunk_bytes=max(chunk_bytes, 1 << 16))
+    _assert_state_equal(state_pack.unpack(header, staging), O.state_dict_round_trip(state))
+
+
+def test_checkpoint_fetched_over_parallel_connections(device):
+    """A payload above 256 MiB is fetched as byte ranges over several connections at once;
+    the result is the sender's state bit for bit, and disallow_checkpoint waits for the
+    requests in flight."""
+    g = torch.Generator(device).manual_seed(1)
+    state = {"user": {"model": {f"w{i}": torch.randn(23_000_000 + i, device=device, generator=g)
+                                for i in range(4)},
+                      "step": 3},
+             "torchft": {"step": 9, "batches_committed": 18}}
+    nbytes = sum(t.numel() * 4 for t in state["user"]["model"].values())
+    assert nbytes > 256 << 20
+    for streams in (1, 3, 4):
+        server = CheckpointServer(timeout=timedelta(seconds=60), fetch_streams=streams)
+        server.send_checkpoint([1], 9, state, timedelta(seconds=60))
+        out = server.recv_checkpoint(0, server.metadata(), 9, timedelta(seconds=60))
+        server.disallow_checkpoint()
+        assert server._readers == 0
+        assert out["torchft"] == state["torchft"] and out["user"]["step"] == 3
+        for k, v in state["user"]["model"].items():
+            assert torch.equal(out["user"]["model"][k], v), (streams, k)
+        with pytest.raises(Exception):  # wrong step: HTTP 400
+            server.allow_checkpoint(10)
+            server.recv_checkpoint(0, server.metadata(), 9, timedelta(seconds=10))
+        server.shutdown()
+
+
 def test_checkpoint_server_with_device_tensors(device):
     """torchft/checkpointing_test.py:17-58 with a tensor payload: the recovering side gets
     the same state, on its GPU, bit for bit."""

@@ -99,3 +99,41 @@ def test_malformed_headers_are_rejected():
         state_pack.parse_header(json.dumps(doc).encode())
     with pytest.raises(ValueError, match="bad magic"):
         state_pack.read_packed(io.BytesIO(b"12345678" + b"\0" * 16), None)
+
+
+def test_peer_supplied_sizes_are_bounded_before_anything_is_allocated():
+    """The header length and the payload size come from the peer: an oversized header length is
+    refused before that many bytes are read, and the entries are validated against the
+    announced payload size before a staging buffer of that size would be allocated."""
+    import struct
+
+    huge = state_pack.MAGIC + struct.pack("<Q", state_pack.MAX_HEADER_BYTES + 1)
+    with pytest.raises(ValueError, match="refused"):
+        state_pack.read_header(io.BytesIO(huge))
+    with pytest.raises(EOFError):
+        state_pack.read_header(io.BytesIO(state_pack.MAGIC + struct.pack("<Q", 100) + b"{}"))
+    with pytest.raises(EOFError):
+        state_pack.read_header(io.BytesIO(state_pack.MAGIC + b"\1\2"))
+    # an entry outside the payload: refused by read_packed before the device is touched
+    doc = {"skeleton": None, "entries": [[1 << 40, 16, "torch.float32", [4], False, False]],
+           "total_bytes": 1 << 20}
+    header = json.dumps(doc).encode()
+    wire = state_pack.MAGIC + struct.pack("<Q", len(header)) + header
+    with pytest.raises(ValueError, match="outside the payload"):
+        state_pack.read_packed(io.BytesIO(wire), None)
+    # validation without decoding the skeleton never unpickles
+    doc = {"skeleton": {"__tft__": "pickle", "type": "x", "data": "AAAA"}, "entries": [], "total_bytes": 0}
+    meta = state_pack.parse_header(json.dumps(doc).encode(), allow_pickle=False, decode_skeleton=False)
+    assert meta["skeleton"] is None and meta["total_bytes"] == 0
+
+
+def test_split_range_covers_the_payload_on_aligned_boundaries():
+    for total in (0, 1, 255, 256, 257, 10_000, (1 << 30) + 123):
+        for parts in (1, 2, 3, 4, 7):
+            ranges = [state_pack.split_range(total, p, parts) for p in range(parts)]
+            assert ranges[0][0] == 0 and ranges[-1][1] == total
+            for (lo, hi), (lo2, _) in zip(ranges, ranges[1:]):
+                assert lo <= hi == lo2
+            assert all(lo % 256 == 0 for lo, hi in ranges if hi > lo)
+    with pytest.raises(ValueError):
+        state_pack.split_range(10, 2, 2)

@@ -33,6 +33,7 @@ import io
 import json
 import pickle
 import struct
+import threading
 from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Any, BinaryIO, Dict, List, Optional, Sequence, Tuple
@@ -278,10 +279,11 @@ def header_total_bytes(header: bytes) -> int:
     return total
 
 
-def parse_header(header: bytes, allow_pickle: bool = True) -> Dict[str, Any]:
+def parse_header(header: bytes, allow_pickle: bool = True, decode_skeleton: bool = True) -> Dict[str, Any]:
     """Decodes a header into ``{"skeleton", "entries", "total_bytes"}``.  Nothing is
     unpickled unless the sender embedded a leaf JSON cannot express and
-    ``allow_pickle`` is true."""
+    ``allow_pickle`` is true.  ``decode_skeleton=False`` only validates the entries
+    (every tensor inside the payload, shapes and byte counts consistent)."""
     try:
         doc = json.loads(header.decode("utf-8"))
     except (UnicodeDecodeError, ValueError) as e:
@@ -301,8 +303,10 @@ def parse_header(header: bytes, allow_pickle: bool = True) -> Dict[str, Any]:
             numel *= x
         if numel * _DTYPES[e.dtype].itemsize != e.nbytes:
             raise ValueError("packed-state header: shape and byte count disagree")
-    return {"skeleton": _decode(doc["skeleton"], allow_pickle), "entries": entries,
-            "total_bytes": total}
+    if total < 0:
+        raise ValueError("packed-state header: negative payload size")
+    skeleton = _decode(doc["skeleton"], allow_pickle) if decode_skeleton else None
+    return {"skeleton": skeleton, "entries": entries, "total_bytes": total}
 
 
 def unpack(
@@ -344,19 +348,138 @@ def unpack(
 
 
 # ---------------------------------------------------------------------------
-# Moving a staging buffer over PCIe and over a byte stream
+# Moving a packed state over PCIe and over a byte stream
 # ---------------------------------------------------------------------------
 
-DEFAULT_CHUNK_BYTES = 256 << 20
+DEFAULT_CHUNK_BYTES = 64 << 20
+MAX_HEADER_BYTES = 256 << 20  # a header is a few hundred bytes per tensor
 
 
-def _pinned(nbytes: int) -> torch.Tensor:
-    return torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+class _PinnedPool:
+    """Pinned host buffers, kept between transfers (pinning a fresh 64 MiB costs tens of
+    milliseconds; a recovery moves tens of gigabytes through a handful of them)."""
+
+    def __init__(self, keep_bytes: int = 2 << 30) -> None:
+        self._lock = threading.Lock()
+        self._free: List[torch.Tensor] = []
+        self._keep_bytes = keep_bytes
+
+    def acquire(self, nbytes: int) -> torch.Tensor:
+        with self._lock:
+            for i, t in enumerate(self._free):
+                if t.numel() >= nbytes:
+                    return self._free.pop(i)
+        return torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+
+    def release(self, t: torch.Tensor) -> None:
+        with self._lock:
+            if sum(x.numel() for x in self._free) + t.numel() <= self._keep_bytes:
+                self._free.append(t)
+
+
+PINNED = _PinnedPool()
+
+
+def split_range(total: int, part: int, parts: int) -> Tuple[int, int]:
+    """Byte range [lo, hi) of ``part`` when a payload of ``total`` bytes is cut into
+    ``parts`` ranges of (almost) equal size on 256-byte boundaries."""
+    if not 0 <= part < parts:
+        raise ValueError(f"part {part} of {parts}")
+    per_part = -(-total // parts)
+    step = -(-per_part // ALIGN) * ALIGN
+    return min(part * step, total), min((part + 1) * step, total)
+
+
+def _pieces(plan: PackPlan, lo: int, hi: int) -> Tuple[List[int], List[torch.Tensor]]:
+    """The tensors' bytes that fall into payload range [lo, hi): (offsets inside the range,
+    byte views of the sources)."""
+    offs: List[int] = []
+    srcs: List[torch.Tensor] = []
+    for e, t in zip(plan.entries, plan.tensors):
+        a, b = max(lo, e.offset), min(hi, e.offset + e.nbytes)
+        if a < b:
+            raw = t.reshape(-1).view(torch.uint8)
+            offs.append(a - lo)
+            srcs.append(raw[a - e.offset : b - e.offset])
+    return offs, srcs
+
+
+def stream_packed(
+    plan: PackPlan,
+    out: BinaryIO,
+    lo: int = 0,
+    hi: Optional[int] = None,
+    chunk_bytes: int = DEFAULT_CHUNK_BYTES,
+    after: Optional["torch.cuda.Event"] = None,
+) -> None:
+    """Writes MAGIC | header length | header | payload bytes [lo, hi) to ``out`` without ever
+    holding more than a few chunks: chunk k+2 is gathered on the device (one launch into a
+    slot of a three-slot ring) while chunk k+1 crosses PCIe into pinned memory and chunk k is
+    written to ``out``.  Device memory: 3 x chunk_bytes; pinned memory: 3 x chunk_bytes.
+    The gather and the device-to-host copies run on two streams of their own, ordered after
+    ``after`` (an event recorded by whoever last wrote the state)."""
+    header = plan.header()
+    out.write(MAGIC)
+    out.write(struct.pack("<Q", len(header)))
+    out.write(header)
+    total = plan.total_bytes
+    hi = total if hi is None else hi
+    if not 0 <= lo <= hi <= total:
+        raise ValueError(f"range [{lo}, {hi}) outside a payload of {total} bytes")
+    if hi == lo or not plan.tensors:
+        return
+    device = plan.tensors[0].device
+    n_slots = 3
+    chunk_bytes = max(ALIGN, min(chunk_bytes, -(-(hi - lo) // ALIGN) * ALIGN))
+    starts = list(range(lo, hi, chunk_bytes))
+    ring = torch.zeros(n_slots * chunk_bytes, dtype=torch.uint8, device=device)
+    slots = [ring[j * chunk_bytes : (j + 1) * chunk_bytes] for j in range(n_slots)]
+    pinned = [PINNED.acquire(chunk_bytes) for _ in range(n_slots)]
+    pack_stream, copy_stream = torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)
+    # the ring was zeroed on the caller's stream
+    ready = torch.cuda.Event()
+    ready.record(torch.cuda.current_stream(device))
+    pack_stream.wait_event(ready)
+    if after is not None:
+        pack_stream.wait_event(after)
+    packed = [torch.cuda.Event() for _ in starts]
+    landed = [torch.cuda.Event() for _ in starts]
+
+    def size(k: int) -> int:
+        return min(chunk_bytes, hi - starts[k])
+
+    try:
+        for k in range(len(starts) + 2):
+            if k < len(starts):  # gather chunk k into its ring slot
+                if k >= n_slots:
+                    pack_stream.wait_event(landed[k - n_slots])  # the slot's last copy left it
+                offs, srcs = _pieces(plan, starts[k], starts[k] + size(k))
+                if srcs:
+                    dsts = [slots[k % n_slots][o : o + s.numel()] for o, s in zip(offs, srcs)]
+                    with torch.cuda.stream(pack_stream):
+                        ops.mt_copy(dsts, srcs)
+                packed[k].record(pack_stream)
+            j = k - 1
+            if 0 <= j < len(starts):  # chunk j crosses PCIe (its pinned slot was written out)
+                copy_stream.wait_event(packed[j])
+                with torch.cuda.stream(copy_stream):
+                    pinned[j % n_slots][: size(j)].copy_(slots[j % n_slots][: size(j)], non_blocking=True)
+                landed[j].record(copy_stream)
+            j = k - 2
+            if 0 <= j < len(starts):  # chunk j goes out
+                landed[j].synchronize()
+                out.write(memoryview(pinned[j % n_slots][: size(j)].numpy()))
+    finally:
+        copy_stream.synchronize()
+        pack_stream.synchronize()
+        for t in pinned:
+            PINNED.release(t)
 
 
 def write_packed(packed: PackedState, out: BinaryIO, chunk_bytes: int = DEFAULT_CHUNK_BYTES) -> None:
-    """Writes the wire layout to ``out``; the payload goes through two pinned bounce
-    buffers so that the copy of chunk k+1 overlaps the write of chunk k."""
+    """Writes the wire layout of an already packed state (a full staging buffer on the
+    device) to ``out``; the payload goes through two pinned bounce buffers so that the copy
+    of chunk k+1 overlaps the write of chunk k."""
     out.write(MAGIC)
     out.write(struct.pack("<Q", len(packed.header)))
     out.write(packed.header)
@@ -367,7 +490,7 @@ def write_packed(packed: PackedState, out: BinaryIO, chunk_bytes: int = DEFAULT_
     assert staging is not None
     stream = torch.cuda.current_stream(staging.device)
     chunk_bytes = min(chunk_bytes, total)
-    bounce = [_pinned(chunk_bytes), _pinned(chunk_bytes)]
+    bounce = [PINNED.acquire(chunk_bytes), PINNED.acquire(chunk_bytes)]
     events = [torch.cuda.Event(), torch.cuda.Event()]
     offsets = list(range(0, total, chunk_bytes))
 
@@ -377,13 +500,18 @@ def write_packed(packed: PackedState, out: BinaryIO, chunk_bytes: int = DEFAULT_
         bounce[i % 2][:n].copy_(staging[lo : lo + n], non_blocking=True)
         events[i % 2].record(stream)
 
-    start(0)
-    for i, lo in enumerate(offsets):
-        n = min(chunk_bytes, total - lo)
-        events[i % 2].synchronize()
-        if i + 1 < len(offsets):
-            start(i + 1)
-        out.write(memoryview(bounce[i % 2][:n].numpy()))
+    try:
+        start(0)
+        for i, lo in enumerate(offsets):
+            n = min(chunk_bytes, total - lo)
+            events[i % 2].synchronize()
+            if i + 1 < len(offsets):
+                start(i + 1)
+            out.write(memoryview(bounce[i % 2][:n].numpy()))
+    finally:
+        stream.synchronize()
+        for t in bounce:
+            PINNED.release(t)
 
 
 def _read_exact(src: BinaryIO, view: memoryview) -> None:
@@ -395,42 +523,95 @@ def _read_exact(src: BinaryIO, view: memoryview) -> None:
         got += n
 
 
+def read_header(src: BinaryIO) -> bytes:
+    """Reads MAGIC | header length | header and returns the header bytes.  The length field
+    comes from the peer: it is bounded before anything of that size is read."""
+    magic = src.read(len(MAGIC))
+    if magic != MAGIC:
+        raise ValueError(f"bad magic {magic!r}: not a packed state")
+    raw = src.read(8)
+    if len(raw) != 8:
+        raise EOFError("stream ended inside the header")
+    (hlen,) = struct.unpack("<Q", raw)
+    if hlen > MAX_HEADER_BYTES:
+        raise ValueError(f"packed-state header of {hlen} bytes: refused (limit {MAX_HEADER_BYTES})")
+    header = src.read(hlen)
+    if len(header) != hlen:
+        raise EOFError("stream ended inside the header")
+    return header
+
+
+def check_payload_fits(header: bytes, device: torch.device) -> int:
+    """Validates the header's entries against its announced payload size, and that size
+    against the device's free memory, BEFORE a staging buffer of that size is allocated;
+    returns the payload size."""
+    total = header_total_bytes(header)
+    parse_header(header, allow_pickle=False, decode_skeleton=False)
+    if total:
+        free, _ = torch.cuda.mem_get_info(device)
+        reusable = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+        if total > free + reusable:
+            raise ValueError(
+                f"packed state announces {total} payload bytes, the device has {free + reusable} free"
+            )
+    return total
+
+
+def read_payload(
+    src: BinaryIO,
+    staging: torch.Tensor,
+    lo: int,
+    hi: int,
+    chunk_bytes: int = DEFAULT_CHUNK_BYTES,
+) -> None:
+    """Receives payload bytes [lo, hi) from ``src`` into ``staging[lo:hi]`` (on the device):
+    chunk by chunk into pinned memory and up to the device as it arrives, on a stream of its
+    own, so host memory use is bounded by two chunks."""
+    if hi <= lo:
+        return
+    device = staging.device
+    stream = torch.cuda.Stream(device=device)
+    chunk_bytes = min(chunk_bytes, hi - lo)
+    bounce = [PINNED.acquire(chunk_bytes), PINNED.acquire(chunk_bytes)]
+    events: List[Optional[torch.cuda.Event]] = [None, None]
+    try:
+        for i, a in enumerate(range(lo, hi, chunk_bytes)):
+            n = min(chunk_bytes, hi - a)
+            ev = events[i % 2]
+            if ev is not None:
+                ev.synchronize()  # the previous upload from this bounce buffer is done
+            _read_exact(src, memoryview(bounce[i % 2][:n].numpy()))
+            with torch.cuda.stream(stream):
+                staging[a : a + n].copy_(bounce[i % 2][:n], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record(stream)
+            events[i % 2] = ev
+    finally:
+        stream.synchronize()
+        for t in bounce:
+            PINNED.release(t)
+
+
 def read_packed(
     src: BinaryIO,
     device: Optional[torch.device],
     chunk_bytes: int = DEFAULT_CHUNK_BYTES,
 ) -> Tuple[bytes, Optional[torch.Tensor]]:
-    """Reads the wire layout; returns ``(header, staging on device)``.  The payload is
-    received chunk by chunk into pinned memory and copied to the device as it arrives,
-    so host memory use is bounded by two chunks."""
-    magic = src.read(len(MAGIC))
-    if magic != MAGIC:
-        raise ValueError(f"bad magic {magic!r}: not a packed state")
-    (hlen,) = struct.unpack("<Q", src.read(8))
-    header = src.read(hlen)
-    if len(header) != hlen:
-        raise EOFError("stream ended inside the header")
+    """Reads the wire layout (whole payload); returns ``(header, staging on device)``."""
+    header = read_header(src)
+    if device is None and torch.cuda.is_available():
+        device = torch.device("cuda", torch.cuda.current_device())
     total = header_total_bytes(header)
+    parse_header(header, allow_pickle=False, decode_skeleton=False)  # before any allocation
     if total == 0:
         return header, None
     if device is None:
-        device = torch.device("cuda", torch.cuda.current_device())
+        raise RuntimeError("the packed state holds device tensors and no GPU is visible")
+    check_payload_fits(header, device)
     staging = torch.empty(total, dtype=torch.uint8, device=device)
-    stream = torch.cuda.current_stream(device)
-    chunk_bytes = min(chunk_bytes, total)
-    bounce = [_pinned(chunk_bytes), _pinned(chunk_bytes)]
-    events: List[Optional[torch.cuda.Event]] = [None, None]
-    for i, lo in enumerate(range(0, total, chunk_bytes)):
-        n = min(chunk_bytes, total - lo)
-        ev = events[i % 2]
-        if ev is not None:
-            ev.synchronize()  # the previous upload from this bounce buffer is done
-        _read_exact(src, memoryview(bounce[i % 2][:n].numpy()))
-        staging[lo : lo + n].copy_(bounce[i % 2][:n], non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record(stream)
-        events[i % 2] = ev
-    stream.synchronize()
+    # the allocation is ordered on the current stream; the upload runs on another
+    torch.cuda.current_stream(device).synchronize()
+    read_payload(src, staging, 0, total, chunk_bytes)
     return header, staging
 
 
