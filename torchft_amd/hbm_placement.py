@@ -50,12 +50,14 @@ from .multi_tensor import current_stream_handle
 logger: logging.Logger = logging.getLogger(__name__)
 
 N_GROUPS = 3
-PROBE_BYTES = 256 << 20      # per buffer and probe: long enough to time, short enough to be free
+PROBE_BYTES = 512 << 20      # per buffer and probe: long enough to time reliably (0.3 ms), short enough to be free
 MIN_PROBE_BYTES = 128 << 20  # tensors below this are not probed (they take their neighbour's group)
 BLOCK_BYTES = 2 << 30        # device memory is taken from torch in blocks of this size
 # probe time / time of a same-group pair: 0.97-1.05 measured inside one group, 0.83-0.85
 # across two (probes of 128 MiB and more)
 SAME_GROUP_RATIO = 0.92
+AMBIGUOUS_BAND = 0.03        # a ratio this close to the threshold is measured again
+RELATIVE_CONTRAST = 1.06     # own-group probe time / next longest, with all three anchors known
 MIN_MODEL_BYTES = 1 << 30    # below this the placement makes no measurable difference
 ALIGN = 256
 
@@ -120,22 +122,39 @@ class GroupMap:
             a = self.anchors[0]
             half = a.numel() // 2 // 16 * 16
             n = min(nbytes, half)
-            t = probe_ms(a[:half], a[half:], n)
+            t = min(probe_ms(a[:half], a[half:], n, repeats=5) for _ in range(2))
             # scale to the requested size if the anchor is shorter than the probe
             self.same_ms[key] = t * (nbytes / n)
         return self.same_ms[key]
 
     def group_of(self, t: torch.Tensor, nbytes: Optional[int] = None) -> Optional[int]:
         """Index of the anchor whose group ``t`` shares, or None if it shares none of the known
-        ones (an unseen group) - or if ``t`` is too small to tell."""
+        ones (an unseen group) - or if ``t`` is too small to tell.
+
+        Once an anchor of every group is known the decision is relative: the probe against
+        the anchor of ``t``'s own group takes clearly longer than against the other two,
+        whatever constant a profiler or a busy host adds to every launch.  Before that, the
+        probe times are compared with the time of a pair that certainly shares a group.
+        An unclear measurement is repeated with more launches."""
         size = _as_bytes(t).numel()
         n = min(size, PROBE_BYTES if nbytes is None else nbytes) // 16 * 16
         if n < MIN_PROBE_BYTES:
             return None
-        same = self._same_ms(n)
-        ratios = [probe_ms(t, anchor, n) / same for anchor in self.anchors]
-        best = max(range(len(ratios)), key=lambda k: ratios[k])
-        return best if ratios[best] > SAME_GROUP_RATIO else None
+        for repeats in (3, 6, 9):
+            times = [probe_ms(t, anchor, n, repeats) for anchor in self.anchors]
+            best = max(range(len(times)), key=lambda k: times[k])
+            if len(self.anchors) >= N_GROUPS:
+                second = max(x for k, x in enumerate(times) if k != best)
+                contrast = times[best] / second
+                if contrast > RELATIVE_CONTRAST:
+                    return best
+                continue  # no anchor stands out: measure again
+            ratio = times[best] / self._same_ms(n)
+            if abs(ratio - SAME_GROUP_RATIO) > AMBIGUOUS_BAND:
+                return best if ratio > SAME_GROUP_RATIO else None
+        if len(self.anchors) >= N_GROUPS:
+            return None
+        return best if ratio > SAME_GROUP_RATIO else None
 
 
 class GroupedPool:
@@ -166,12 +185,21 @@ class GroupedPool:
         for piece in (storage[:PROBE_BYTES], storage[n - PROBE_BYTES:]):
             g = m.group_of(piece)
             if g is None:
-                if len(m.anchors) >= N_GROUPS:
+                if len(m.anchors) >= N_GROUPS or not self._clearly_new(storage):
                     return None  # matches no group clearly: leave it alone
                 m.anchors.append(piece)
                 g = len(m.anchors) - 1
             ends.append(g)
         return ends[0] if ends[0] == ends[1] else None
+
+    def _clearly_new(self, storage: torch.Tensor) -> bool:
+        """A second, longer measurement before a block founds a new group: an anchor that in
+        truth lies in a known group would make every later block of that group unclassifiable."""
+        m = self.map
+        n = min(storage.numel(), 2 * PROBE_BYTES) // 16 * 16
+        same = m._same_ms(n)
+        return all(probe_ms(storage, anchor, n, repeats=9) / same < SAME_GROUP_RATIO - AMBIGUOUS_BAND
+                   for anchor in m.anchors)
 
     def free_bytes(self, group: int) -> int:
         return sum(b.free() for b in self.blocks if b.group == group)
@@ -213,6 +241,11 @@ class GroupedPool:
                     b.used = start + nbytes
                     return b.storage[start:start + nbytes]
         return None
+
+    def reset(self) -> None:
+        """Forgets everything handed out (the caller has dropped those tensors)."""
+        for b in self.blocks:
+            b.used = 0
 
     def release_unused(self) -> None:
         """Gives every block nothing was taken from back to the device."""
@@ -257,6 +290,17 @@ def allocate_apart(
     sizes = [t.numel() * t.element_size() for t in like]
     if sum(sizes) < MIN_MODEL_BYTES:
         return None
+    try:
+        return _allocate_apart(like, sizes, n_copies, device)
+    except Exception as e:  # placement is an optimisation: never let it fail an allocation
+        logger.warning("hbm placement gave up (%s); default allocation", e)
+        torch.cuda.empty_cache()
+        return None
+
+
+def _allocate_apart(
+    like: Sequence[torch.Tensor], sizes: List[int], n_copies: int, device: torch.device
+) -> Optional[List[List[torch.Tensor]]]:
     torch.cuda.synchronize(device)
     pool = GroupedPool(device)
     largest = max(sizes)
@@ -282,7 +326,7 @@ def allocate_apart(
     pool.grow_until(lambda pl: all(pl.free_bytes(g) >= n for g, n in need.items()), block_bytes=block)
     copies: List[List[torch.Tensor]] = [[] for _ in range(n_copies)]
     order = sorted(range(len(like)), key=lambda i: -sizes[i])  # large tensors first: they pack better
-    placed: Dict[Tuple[int, int], torch.Tensor] = {}
+    placed: Dict[Tuple[int, int], Optional[torch.Tensor]] = {}
     misplaced = 0
     for i in order:
         for k in range(n_copies):
@@ -292,12 +336,16 @@ def allocate_apart(
             if raw is None and sizes[i]:
                 raw = pool.take(sizes[i], others)
                 misplaced += 1
-            if raw is None:
-                raw = torch.empty(max(sizes[i], 1), dtype=torch.uint8, device=device)[:sizes[i]]
-            placed[(i, k)] = raw.view(like[i].dtype).view(like[i].shape)
+            placed[(i, k)] = raw
+    # everything the search held but did not use goes back BEFORE anything else is allocated:
+    # what found no room in the pool must not fail for memory the pool itself is sitting on
+    pool.release_unused()
+    for (i, k), raw in list(placed.items()):
+        if raw is None:
+            raw = torch.empty(max(sizes[i], 1), dtype=torch.uint8, device=device)[: sizes[i]]
+        placed[(i, k)] = raw.view(like[i].dtype).view(like[i].shape)
     for k in range(n_copies):
         copies[k] = [placed[(i, k)] for i in range(len(like))]
-    pool.release_unused()
     logger.info(
         "hbm placement: %d tensors x %d copies over %d bank groups (%d not in their preferred group)",
         len(like), n_copies, n_groups, misplaced,
