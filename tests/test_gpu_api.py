@@ -177,16 +177,20 @@ def test_localsgd_mlp_two_replicas(device):
     optimizer = optim.SGD(model.parameters(), lr=1e-3)
     with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
         backup0 = cpu(lsgd._backup_parameters.values())
+        seen = {}
+        perform = lsgd._perform_sync
+
+        def recording_perform_sync():  # what the sync sees: the parameters after the local step
+            seen["local"] = cpu(p.data for p in model.parameters())
+            perform()
+
+        lsgd._perform_sync = recording_perform_sync
         model(torch.randn(4, 1024, device=device)).square().mean().backward()
         optimizer.step()  # local step, then the sync fires from the post hook
-        # reconstruct what the sync saw: parameters after the local step
-        local = [b - 1e-3 * p.grad.cpu() for b, p in zip(backup0, model.parameters())]
-        want = O.localsgd_perform_sync([local, cpu(q.data for q in peers[0].parameters())],
+        want = O.localsgd_perform_sync([seen["local"], cpu(q.data for q in peers[0].parameters())],
                                        backup0, [True, True], 2, True)
         for p, w, (name, b) in zip(model.parameters(), want["params"], lsgd._backup_parameters.items()):
-            # the local SGD step itself is torch's (GPU fma vs CPU fma may differ by an ulp),
-            # so this leg is held to the specified fp32 tolerance, not to bit equality
-            torch.testing.assert_close(p.data.cpu(), w, rtol=RTOL_F32, atol=1e-9)
+            assert_bits_equal(p.data, w, f"params {name}")
             assert_bits_equal(b, p.data, f"backup {name} == params after commit")
     assert manager.current_step() == 1
     manager.shutdown(wait=False)

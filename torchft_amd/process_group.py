@@ -86,30 +86,21 @@ class ProcessGroupDummy(ProcessGroup):
         assert world == 1
         self._rank = rank
         self._world = world
-        self.wait_count = 0
-        self.get_future_count = 0
-        self._work: List[Work] = []
         self.configure_count = 0
 
     def configure(self, store_addr: str, rank: int, world_size: int) -> None:
         self.configure_count += 1
 
     def broadcast(self, tensor_list, opts) -> Work:  # type: ignore[override]
-        res = _DummyWork(tensor_list)
-        self._work.append(res)
-        return res
+        return _DummyWork(tensor_list)
 
     def allgather(self, output_tensors, input_tensor, opts) -> Work:  # type: ignore[override]
         for o, i in zip(output_tensors[0], input_tensor):
             o.copy_(i)
-        res = _DummyWork(output_tensors)
-        self._work.append(res)
-        return res
+        return _DummyWork(output_tensors)
 
     def allreduce(self, tensors, opts) -> Work:  # type: ignore[override]
-        res = _DummyWork(tensors)
-        self._work.append(res)
-        return res
+        return _DummyWork(tensors)
 
     def size(self) -> int:
         return self._world
