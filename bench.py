@@ -39,7 +39,7 @@ LR, MOMENTUM = 0.7, 0.9
 HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo"
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
              "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
-             "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice"]
+             "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -62,9 +62,14 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--layout", default="",
                     help="comma list: alias_p (DiLoCo workloads: the live parameters are replica 0, "
                          "updated in place), flat_backup / flat_momentum (backup / momentum tensors are "
-                         "views of one flat allocation, back to back without padding), no_placement "
+                         "views of one flat allocation, back to back without padding), misaligned (DiLoCo "
+                         "workloads: every tensor re-allocated to start 4 bytes past a 16-byte boundary; moved: "
+                         "the same re-allocation, 16 bytes past, as the aligned control), no_placement "
                          "(the library allocates backup / momentum / pseudo-gradients without looking "
                          "at HBM bank groups)")
+    ap.add_argument("--storage-dtype", choices=("f32", "bf16"), default="f32",
+                    help="DiLoCo workloads: dtype of parameters, backup, momentum and replicas "
+                         "(arithmetic is fp32 either way; the named configurations are f32)")
     ap.add_argument("--arena", action="store_true",
                     help="carve all tensors of the DiLoCo workload out of one device allocation "
                          "instead of allocating each separately (makes no measurable difference)")
@@ -188,6 +193,10 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         shapes, n_rep = workloads.llama3_8b_shapes(), 2
     else:
         shapes, n_rep = workloads.gpt2_small_shapes(), 4
+    dtype = torch.bfloat16 if args.storage_dtype == "bf16" else torch.float32
+    esize = 2 if dtype == torch.bfloat16 else 4
+    if args.arena and dtype != torch.float32:
+        raise SystemExit("--arena is an fp32 layout experiment")
     if args.arena:
         per_set = sum(-(-workloads.numel(sh) * 4 // 256) * 256 for _, sh in shapes)
         arena = torch.empty((3 + n_rep) * per_set, dtype=torch.uint8, device=dev)
@@ -211,16 +220,34 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         bufs = carve(workloads.normal_tensors(shapes, 1e-3, 4000, dev))
         torch.cuda.empty_cache()
     else:
-        wl = workloads.make_diloco_workload(shapes, n_rep, dev)
+        wl = workloads.make_diloco_workload(shapes, n_rep, dev, dtype)
         params = [torch.empty_like(t) for t in wl.backup]
-        bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev)
+        bufs = workloads.normal_tensors(shapes, 1e-3, 4000, dev, dtype)
     layout = [x for x in args.layout.split(",") if x]
+    if "misaligned" in layout or "moved" in layout:
+        # misaligned: every tensor of every stream starts one element (4 bytes) past a 16-byte
+        # boundary; moved: the same re-allocation with a shift of 16 bytes (the aligned control)
+        first = 1 if "misaligned" in layout else 16 // esize
+
+        def shifted(ts):
+            for i, t in enumerate(ts):
+                moved = torch.empty(t.numel() + 16, dtype=t.dtype, device=dev)[first:first + t.numel()].view(t.shape)
+                moved.copy_(t)
+                ts[i] = moved
+            return ts
+
+        for ts in (wl.backup, bufs, params, *wl.replicas):
+            shifted(ts)
+        torch.cuda.empty_cache()
+        assert all(t.data_ptr() % 16 == (esize * first) % 16 for t in params + wl.backup + bufs)
     for item in layout:
+        if item in ("misaligned", "moved"):
+            continue
         if item == "alias_p":
             params = wl.replicas[0]
         elif item in ("flat_backup", "flat_momentum"):
             src = wl.backup if item == "flat_backup" else bufs
-            flat = torch.empty(sum(t.numel() for t in src), dtype=torch.float32, device=dev)
+            flat = torch.empty(sum(t.numel() for t in src), dtype=dtype, device=dev)
             views = ops.flat_views(flat, src)
             ops.mt_copy(views, src)
             torch.cuda.synchronize()
@@ -264,25 +291,26 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
 
     wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
     for probe in (0, len(params) // 2, len(params) - 1):
-        same = torch.equal(params[probe].view(torch.int32), wl.backup[probe].view(torch.int32))
+        same = torch.equal(params[probe].view(torch.uint8), wl.backup[probe].view(torch.uint8))
         if not same or not torch.isfinite(params[probe]).all():
             raise RuntimeError("output check failed: parameters are not finite or differ from the backup")
 
     n_params = wl.n_params
     # read N replicas, backup, momentum; write momentum, parameters, backup
-    algo_bytes = n_params * (4 * n_rep + 20)
+    algo_bytes = n_params * esize * (n_rep + 5)
     out = base_line(
         args, HEADLINE_METRIC if which == "llama3_8b" else "outer-sync params/sec, GPT-2-small DiLoCo",
         n_params / (wall_ms * 1e-3), "params/s", wall_ms, "f32",
-        {"workload": f"DiLoCo outer step, fp32, {which}-shaped params ({len(shapes)} tensors, "
+        {"workload": f"DiLoCo outer step, {'fp32' if esize == 4 else 'bf16 storage with fp32 arithmetic'}, {which}-shaped params ({len(shapes)} tensors, "
                      f"{n_params} params), {n_rep} simulated replicas, Nesterov SGD lr={LR} "
                      f"momentum={MOMENTUM}, one fused multi-tensor launch per step",
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
          "allocation": ("every tensor is a contiguous view carved out of one device allocation"
                         if args.arena else "one device allocation per tensor"),
          "layout": layout})
-    out["roofline"] = roofline(algo_bytes, kernel_ms, f"mt_stream_kernel<F32, DilocoFusedOp<{n_rep}>>",
-                               workload=f"diloco_{which}")
+    out["roofline"] = roofline(algo_bytes, kernel_ms,
+                               f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<{n_rep}>>",
+                               workload=f"diloco_{which}" if esize == 4 else f"diloco_{which}_bf16")
     if reseeds[0]:
         out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]
         out["roofline"]["note"] = ("steps that re-seed the state include two extra copy launches in "
@@ -307,12 +335,14 @@ def bench_diloco_api(args) -> Dict[str, object]:
 
     dev = torch.device("cuda", 0)
     shapes = workloads.llama3_8b_shapes()
+    dtype = torch.bfloat16 if args.storage_dtype == "bf16" else torch.float32
+    esize = 2 if dtype == torch.bfloat16 else 4
 
     class Bag(nn.Module):
         def __init__(self) -> None:
             super().__init__()
             self.ps = nn.ParameterList(
-                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev)])
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev, dtype)])
 
     model = Bag()
     peer = workloads.drifted_replica([p.data for p in model.parameters()], 1e-3, 1001)
@@ -332,12 +362,14 @@ def bench_diloco_api(args) -> Dict[str, object]:
     manager.shutdown(wait=False)
     out = base_line(args, HEADLINE_METRIC + " (through DiLoCo.sync())", n_params / (wall_ms * 1e-3),
                     "params/s", wall_ms, "f32",
-                    {"workload": "DiLoCo.sync() on a module with the 291 Llama-3-8B fp32 parameters, "
+                    {"workload": "DiLoCo.sync() on a module with the 291 Llama-3-8B "
+                                 f"{'fp32' if esize == 4 else 'bf16'} parameters, "
                                  "Manager + ProcessGroupLocalReplicas(world 2), outer torch.optim.SGD "
                                  "Nesterov; parameters updated in place (the live parameters are "
                                  "replica 0)",
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
-    out["roofline"] = roofline(n_params * 28, kernel_ms, "mt_stream_kernel<F32, DilocoFusedOp<2>>")
+    out["roofline"] = roofline(n_params * 7 * esize, kernel_ms,
+                               f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<2>>")
     out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
     return out
 
@@ -517,6 +549,99 @@ def bench_localsgd(args) -> Dict[str, object]:
             "sample": f"{args.cpu_layers} of 32 decoder layers (no embeddings), {args.cpu_steps} steps after "
                       f"1 warm-up; {n_cpu} params, {dt * 1e3:.1f} ms/step; per-tensor torch CPU ops "
                       f"(sum of replicas, divide, backup copy)"}
+    return out
+
+
+def bench_host_backup(args) -> Dict[str, object]:
+    """LocalSGD's backup in pinned host memory (the reference's default placement): how long
+    the training stream is held up by a save, and whether the transfer really overlaps
+    compute.  The reference issues one copy per tensor on the training stream
+    (torchft/local_sgd.py:121-125, with a TODO to use a separate stream); here one gather
+    launch runs on the training stream and one PCIe transfer on a side stream."""
+    from torchft_amd import ops, workloads
+    from torchft_amd.local_sgd import _PackedHostBackup
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes(args.cpu_layers * 2, with_embeddings=False)
+    params = workloads.normal_tensors(shapes, 0.02, workloads.SEED_BACKUP, dev)
+    other = workloads.drifted_replica(params, 1e-3, workloads.SEED_REPLICA)
+    out_t = [torch.empty_like(t) for t in params]
+    n_params = sum(t.numel() for t in params)
+    nbytes = 4 * n_params
+    backup = _PackedHostBackup([(str(i), t) for i, t in enumerate(params)], pin_memory=True)
+    stream = torch.cuda.current_stream(dev)
+
+    def ev():
+        return torch.cuda.Event(enable_timing=True)
+
+    cached = [None]
+
+    def compute():  # stand-in for the next inner steps: an HBM-bound launch over the model
+        cached[0] = ops.mt_reduce_avg([out_t], [params, other], 0b11, 2, table=cached[0])
+
+    for _ in range(2):
+        compute()
+    torch.cuda.synchronize()
+    a, b = ev(), ev()
+    a.record()
+    for _ in range(10):
+        compute()
+    b.record()
+    torch.cuda.synchronize()
+    compute_alone_ms = a.elapsed_time(b) / 10
+
+    held, total, overlapped = [], [], []
+    for it in range(args.warmup + args.steps):
+        torch.cuda.synchronize()
+        a, b, c = ev(), ev(), ev()
+        t0 = time.perf_counter()
+        a.record()
+        backup.save(params)
+        b.record()
+        for _ in range(10):
+            compute()
+        c.record()
+        backup.wait()
+        t_host = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
+        if it >= args.warmup:
+            held.append(a.elapsed_time(b))
+            total.append(t_host)
+            overlapped.append(b.elapsed_time(c) / 10)
+    for i in (0, len(params) // 2, len(params) - 1):
+        if not torch.equal(backup.host_views[i], params[i].cpu()):
+            raise RuntimeError("output check failed: the host backup differs from the parameters")
+
+    # the reference's form: one copy per tensor into the pinned tensors, on the training stream
+    per_tensor = []
+    for it in range(2 + 3):
+        torch.cuda.synchronize()
+        a, b = ev(), ev()
+        a.record()
+        for h, p in zip(backup.host_views, params):
+            h.copy_(p, non_blocking=True)
+        b.record()
+        torch.cuda.synchronize()
+        if it >= 2:
+            per_tensor.append(a.elapsed_time(b))
+    mean = lambda xs: sum(xs) / len(xs)
+    held_ms, total_ms = mean(held), mean(total)
+    out = base_line(
+        args, "LocalSGD host backup: bytes saved per second of training-stream time", nbytes / (held_ms * 1e-3) / 1e9,
+        "GB/s", held_ms, "u8",
+        {"workload": f"save of {len(shapes)} fp32 tensors ({n_params} params, {nbytes / 1e9:.1f} GB; "
+                     f"{args.cpu_layers * 2} of 32 Llama-3-8B decoder layers) into pinned host memory: one "
+                     "gather launch on the training stream, one transfer on a side stream",
+         "n_tensors": len(shapes), "n_params": n_params})
+    out["roofline"] = roofline(2 * nbytes, held_ms, "mt_copy_kernel")
+    out["host_backup"] = {
+        "training_stream_held_ms": held_ms,
+        "save_complete_on_host_ms": total_ms,
+        "pcie_GBps": nbytes / (total_ms * 1e-3) / 1e9,
+        "compute_launch_alone_ms": compute_alone_ms,
+        "compute_launch_during_transfer_ms": mean(overlapped),
+        "per_tensor_copies_on_training_stream_ms": mean(per_tensor),
+    }
     return out
 
 
@@ -740,6 +865,8 @@ def main() -> int:
         out = bench_diloco_two_phase(args)
     elif args.workload == "placement_llama3_8b_slice":
         out = bench_placement(args)
+    elif args.workload == "host_backup_llama3_8b":
+        out = bench_host_backup(args)
     else:
         out = bench_localsgd(args)
     print(json.dumps(out), flush=True)

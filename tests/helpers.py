@@ -21,3 +21,15 @@ def assert_bits_equal(actual: torch.Tensor, expected: torch.Tensor, what: str = 
             f"got {actual.detach().cpu().reshape(-1)[i].item()!r}, "
             f"expected {expected.detach().cpu().reshape(-1)[i].item()!r}"
         )
+
+
+def assert_bits_equal_up_to_nan_payload(actual: torch.Tensor, expected: torch.Tensor, what: str = "") -> None:
+    """Bit equality wherever the expected value is a number; where it is a NaN the actual
+    value must be a NaN too (which NaN an operation returns is not part of IEEE 754's
+    required behaviour and differs between the host's and the GPU's arithmetic)."""
+    a, e = actual.detach().cpu().reshape(-1), expected.detach().cpu().reshape(-1)
+    assert a.shape == e.shape, f"{what}: shape {tuple(a.shape)} vs {tuple(e.shape)}"
+    nan = torch.isnan(e.float())
+    assert torch.equal(torch.isnan(a.float()), nan), f"{what}: NaNs are not where the checker has them"
+    keep = ~nan
+    assert_bits_equal(a[keep], e[keep], what)

@@ -11,7 +11,7 @@ import itertools
 import pytest
 import torch
 
-from helpers import assert_bits_equal
+from helpers import assert_bits_equal, assert_bits_equal_up_to_nan_payload
 from oracle import replica_sync as O
 from torchft_amd import ops, workloads
 
@@ -440,3 +440,76 @@ def test_fp16_result_is_rounded_from_the_fp32_value(device):
     assert_bits_equal(p_d, want["params"][0])
     assert_bits_equal(b_d, want["backup"][0])
     assert_bits_equal(m_d, want["momentum"][0])
+
+
+def _bit_patterns(n, dtype, seed):
+    """Values over the whole encoding: random bit patterns, plus runs confined to the
+    smallest exponents (denormal and barely normal), the largest ones (next to overflow,
+    infinities, NaNs) and ordinary magnitudes."""
+    g = torch.Generator().manual_seed(seed)
+    if dtype == torch.float32:
+        raw = torch.randint(-2**31, 2**31, (n,), generator=g, dtype=torch.int64).to(torch.int32)
+        mant, sign, shift, top = 0x007fffff, -2**31, 23, 0xff
+    else:
+        raw = torch.randint(-2**15, 2**15, (n,), generator=g, dtype=torch.int64).to(torch.int16)
+        shift = 7 if dtype == torch.bfloat16 else 10
+        mant, sign, top = (1 << shift) - 1, -2**15, 0xff if dtype == torch.bfloat16 else 0x1f
+    kind = torch.randint(0, 4, (n,), generator=g)
+    low = torch.randint(0, 3, (n,), generator=g, dtype=torch.int64)
+    high = top - torch.randint(0, 3, (n,), generator=g, dtype=torch.int64)
+    r64 = raw.to(torch.int64)
+    keep = r64 & (mant | sign)
+    r64 = torch.where(kind == 1, keep | (low << shift), r64)
+    r64 = torch.where(kind == 2, keep | (high << shift), r64)
+    out = r64.to(raw.dtype).view(dtype)
+    ordinary = torch.randn(n, generator=g).to(dtype)
+    return torch.where(kind == 3, ordinary, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n_replicas,mask,nump", [(2, 0b11, 2), (2, 0b11, 1), (4, 0b1111, 4), (3, 0b111, 3),
+                                                 (2, 0b01, 2), (8, 0xFF, 8), (2, 0b11, 64)])
+def test_reduce_avg_over_the_whole_encoding(device, dtype, n_replicas, mask, nump):
+    """Denormals, values next to overflow, infinities and NaNs through the reduction, for
+    divisors that are powers of two (multiplied by the exact reciprocal when everybody
+    participates) and divisors that are not (IEEE division), on full and ragged slabs."""
+    numel = 3 * 65536 + 1234
+    reps = [_bit_patterns(numel, dtype, 900 + r) for r in range(n_replicas)]
+    want = O.manager_allreduce_(reps, mask_to_list(mask, n_replicas), nump, torch.float32)
+    out = torch.empty(numel, dtype=dtype, device=device)
+    ops.reduce_avg_(out, [r.to(device) for r in reps], mask, nump)
+    assert_bits_equal_up_to_nan_payload(out, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sgd_kw", [SGD_CASES[0], SGD_CASES[2]])
+@pytest.mark.parametrize("n_replicas,mask,nump", [(2, 0b11, 2), (2, 0b11, 3), (4, 0b0111, 4)])
+def test_diloco_over_the_whole_encoding(device, dtype, sgd_kw, n_replicas, mask, nump):
+    """The fused step and the two-launch form on inputs drawn over the whole encoding, in
+    the common configuration (everybody participates, power-of-two divisor, Nesterov
+    momentum) and outside it."""
+    numel = 2 * 65536 + 777
+    sgd = ops.OuterSGD(**sgd_kw)
+    kw = dict(lr=sgd.lr, momentum=sgd.momentum, dampening=sgd.dampening,
+              weight_decay=sgd.weight_decay, nesterov=sgd.nesterov)
+    flags = mask_to_list(mask, n_replicas)
+    backup = [_bit_patterns(numel, dtype, 1)]
+    bufs = [_bit_patterns(numel, dtype, 2)]
+    reps = [[_bit_patterns(numel, dtype, 10 + r)] for r in range(n_replicas)]
+    extra = {} if dtype == torch.float32 else dict(accumulate_dtype=torch.float32)
+    want = O.diloco_perform_sync(reps, backup, bufs, flags, nump, True, **kw, **extra)
+    to_dev = lambda ts: [t.to(device) for t in ts]
+    b_d, m_d, r_d = to_dev(backup), to_dev(bufs), [to_dev(r) for r in reps]
+    p_d = [torch.empty_like(b_d[0])]
+    ops.mt_diloco_outer(p_d, b_d, m_d, r_d, sgd, False, mask, nump)
+    assert_bits_equal_up_to_nan_payload(p_d[0], want["params"][0], "params")
+    assert_bits_equal_up_to_nan_payload(b_d[0], want["backup"][0], "backup")
+    assert_bits_equal_up_to_nan_payload(m_d[0], want["momentum"][0], "momentum")
+    if dtype == torch.float32:  # two launches, the pseudo-gradient passing through memory
+        b_d, m_d = to_dev(backup), to_dev(bufs)
+        g_d = [torch.empty_like(b_d[0])]
+        ops.mt_pseudograd_avg(g_d, p_d, b_d, r_d, True, mask, nump)
+        assert_bits_equal_up_to_nan_payload(g_d[0], want["grads"][0], "grads")
+        ops.mt_outer_sgd(p_d, b_d, m_d, g_d, sgd, False)
+        assert_bits_equal_up_to_nan_payload(p_d[0], want["params"][0], "two-launch params")
+        assert_bits_equal_up_to_nan_payload(m_d[0], want["momentum"][0], "two-launch momentum")

@@ -416,6 +416,200 @@ def test_heal_applies_the_recovered_state(cpu_ops):
     server.shutdown()
 
 
+def _reference_quorum(**kw) -> QuorumResult:
+    """The quorum the reference's manager tests script (torchft/manager_test.py:134-145)."""
+    base = dict(quorum_id=123, replica_rank=1, replica_world_size=2, max_step=1, max_rank=1,
+                max_world_size=2, heal=False, recover_src_manager_address="manager address")
+    base.update(kw)
+    return QuorumResult(**base)
+
+
+class _TimedQuorum(ScriptedQuorum):
+    """Records the time-outs the Manager passes on."""
+
+    def __init__(self, result):
+        super().__init__(result)
+        self.quorum_timeouts, self.commit_timeouts = [], []
+
+    def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+        self.quorum_timeouts.append(timeout)
+        return super().quorum(rank, step, checkpoint_metadata, shrink_only, timeout)
+
+    def should_commit(self, rank, step, should_commit, timeout):
+        self.commit_timeouts.append(timeout)
+        return super().should_commit(rank, step, should_commit, timeout)
+
+
+def _healing_manager(quorum: QuorumResult, **kw):
+    """A Manager whose own checkpoint server also plays the healthy peer, as the
+    reference's healing tests arrange it (torchft/manager_test.py:181-190)."""
+    loaded = MagicMock()
+    transport = CheckpointServer(timeout=timedelta(seconds=10))
+
+    class Client(ScriptedQuorum):
+        def checkpoint_metadata(self, address, rank, timeout):
+            assert address == "manager address"
+            return transport.metadata()
+
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=loaded, state_dict=lambda: {},
+                quorum_client=Client(quorum), checkpoint_transport=transport, **kw)
+    m._pg.allreduce.return_value = _DummyWork(None)
+    transport.send_checkpoint(dst_ranks=[], step=quorum.max_step, state_dict=m._manager_state_dict(),
+                              timeout=timedelta(seconds=10))
+    return m, loaded
+
+
+def test_state_dict_and_user_state_dict():
+    """torchft/manager_test.py:76-127."""
+    load = MagicMock()
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=load, state_dict=lambda: {},
+                min_replica_size=2, quorum_client=ScriptedQuorum(_reference_quorum()))
+    assert m.state_dict() == {"step": 0, "batches_committed": 0}
+    assert m._manager_state_dict() == {"user": {}, "torchft": {"step": 0, "batches_committed": 0}}
+    m.set_state_dict_fns(load, lambda: {"new_state": 1})
+    assert m._manager_state_dict() == {"user": {"new_state": 1},
+                                       "torchft": {"step": 0, "batches_committed": 0}}
+    m.load_state_dict({"step": 1234, "batches_committed": 2345})
+    assert m.current_step() == 1234 and m.batches_committed() == 2345
+    m.shutdown(wait=False)
+
+
+def test_quorum_happy(cpu_ops):
+    """torchft/manager_test.py:129-163."""
+    m = _manager(quorum=ScriptedQuorum(_reference_quorum()))
+    m._pg.allreduce.return_value = _DummyWork(None)
+    assert m._quorum_id == -1 and m.current_step() == 0 and m.batches_committed() == 0
+    m.start_quorum()
+    m.allreduce(torch.tensor([1.0])).wait()
+    assert len(m._pending_work) == 1
+    assert m.should_commit()
+    assert len(m._pending_work) == 0
+    assert m._quorum_id == 123 and m.current_step() == 1
+    assert m._pg.allreduce.call_count == 1
+    m.start_quorum()
+    assert m.batches_committed() == 2
+    m.shutdown(wait=False)
+
+
+def test_quorum_heal_sync(cpu_ops):
+    """torchft/manager_test.py:165-212: with a synchronous quorum the recovered state is
+    applied before the step, and the healed replica takes part in it."""
+    q = _reference_quorum(max_step=20, max_rank=None, heal=True, recover_src_rank=0)
+    m, loaded = _healing_manager(q, min_replica_size=2, use_async_quorum=False)
+    assert m._quorum_id == -1 and m.current_step() == 0
+    m.start_quorum()
+    m.allreduce(torch.tensor([1.0])).wait()
+    assert not m._healing
+    assert m.is_participating() and m.num_participants() == 2
+    assert m.should_commit()
+    assert m._quorum_id == 123 and m.current_step() == 21
+    assert m._pg.allreduce.call_count == 1
+    assert loaded.call_count == 1
+    m.shutdown(wait=False)
+
+
+def test_quorum_heal_async_not_enough_participants(cpu_ops):
+    """torchft/manager_test.py:214-276: a healing replica contributes zeros, and a step
+    with fewer up-to-date replicas than min_replica_size does not commit."""
+    q = _reference_quorum(max_step=20, max_rank=None, max_world_size=1, heal=True, recover_src_rank=0)
+    m, loaded = _healing_manager(q, min_replica_size=2, use_async_quorum=True)
+    m.start_quorum()
+    m._quorum_future.result()
+    assert m._healing and not m.is_participating() and m.num_participants() == 1
+    grad = torch.tensor([1.0])
+    m.allreduce(grad).wait()
+    torch.testing.assert_close(grad, torch.zeros_like(grad))
+    assert not m.should_commit()
+    assert m.current_step() == 20 and m._quorum_id == 123
+    assert m._pg.allreduce.call_count == 1
+    assert loaded.call_count == 1
+    q.heal = False
+    m.start_quorum()
+    assert m.current_step() == 20 and m.batches_committed() == 0
+    m.shutdown(wait=False)
+
+
+def test_quorum_heal_async_zero_grad(cpu_ops):
+    """torchft/manager_test.py:278-336."""
+    q = _reference_quorum(max_step=20, max_rank=None, max_world_size=1, heal=True, recover_src_rank=0)
+    m, loaded = _healing_manager(q, min_replica_size=1, use_async_quorum=True)
+    m.start_quorum()
+    m._quorum_future.result()
+    assert m._healing
+    grad = torch.tensor([1.0])
+    m.allreduce(grad).wait()
+    torch.testing.assert_close(grad, torch.zeros_like(grad))
+    assert m.should_commit()
+    assert m.num_participants() == 1 and m.current_step() == 21
+    assert m._quorum_id == 123 and m._pg.allreduce.call_count == 1
+    assert loaded.call_count == 1
+    q.heal = False
+    m.start_quorum()
+    assert m.current_step() == 21 and m.batches_committed() == 1
+    m.shutdown(wait=False)
+
+
+def test_quorum_no_healing(cpu_ops):
+    """torchft/manager_test.py:444-476: ``allow_heal=False`` neither fetches a checkpoint
+    nor takes part, but the step is still counted with the up-to-date replicas."""
+    q = _reference_quorum(replica_rank=0, replica_world_size=3, max_rank=None, max_world_size=2,
+                          heal=True, recover_src_rank=1)
+    client = ScriptedQuorum(q)
+    client.checkpoint_metadata = MagicMock(side_effect=AssertionError("must not heal"))
+    m = _manager(quorum=client, min_replica_size=2)
+    m._pg.allreduce.return_value = _DummyWork(None)
+    m.start_quorum(allow_heal=False)
+    m.allreduce(torch.tensor([1.0])).wait()
+    assert not m.is_participating() and m.num_participants() == 2
+    assert m.should_commit()
+    assert m.batches_committed() == 2 and m.current_step() == 1
+    m.shutdown(wait=False)
+
+
+def test_manager_report_error():
+    """torchft/manager_test.py:478-485."""
+    m = _manager()
+    assert m.errored() is None
+    e = RuntimeError("some error")
+    m.report_error(e)
+    assert m.errored() is e
+    m.shutdown(wait=False)
+
+
+def test_quorum_happy_timeouts(cpu_ops):
+    """torchft/manager_test.py:545-575: per-call time-outs reach the quorum client."""
+    client = _TimedQuorum(_reference_quorum())
+    m = _manager(quorum=client, use_async_quorum=False, timeout=timedelta(seconds=10),
+                 quorum_timeout=timedelta(seconds=60))
+    m.start_quorum(timeout=timedelta(seconds=12))
+    assert client.quorum_timeouts[-1] == timedelta(seconds=12)
+    assert m.should_commit(timeout=timedelta(seconds=23))
+    assert client.commit_timeouts[-1] == timedelta(seconds=23)
+    m.start_quorum()
+    assert client.quorum_timeouts[-1] == timedelta(seconds=60)
+    assert m.should_commit()
+    assert client.commit_timeouts[-1] == timedelta(seconds=10)
+    m.shutdown(wait=False)
+
+
+def test_quorum_timeout():
+    """torchft/manager_integ_test.py:621-660: one replica of a two-replica lighthouse gives
+    up after the time-out it was given, for the quorum and for the commit vote alike."""
+    import time
+
+    from torchft_amd import InProcessLighthouse
+
+    lighthouse = InProcessLighthouse(min_replicas=2)
+    m = Manager(pg=create_autospec(ProcessGroup), load_state_dict=lambda x: None, state_dict=lambda: None,
+                min_replica_size=2, use_async_quorum=False, rank=0, world_size=2,
+                quorum_client=lighthouse.client("lonely"))
+    t0 = time.monotonic()
+    with pytest.raises(TimeoutError, match="quorum did not form within"):
+        m.start_quorum(timeout=timedelta(seconds=0.01))
+    assert time.monotonic() - t0 < 1.0
+    m.shutdown(wait=False)
+
+
 # ---------------------------------------------------------------------------
 # Local replica group
 # ---------------------------------------------------------------------------

@@ -69,7 +69,7 @@ struct F32 {
 
 __device__ inline uint32_t f32_to_bf16_bits(float f) {
   // round to nearest even; NaN collapses to the canonical quiet NaN (what
-  // c10::BFloat16 does on the host)
+  // c10::BFloat16's scalar conversion does on the host)
   uint32_t u = __float_as_uint(f);
   if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
   u += 0x7fffu + ((u >> 16) & 1u);
@@ -86,11 +86,19 @@ struct BF16 {
       v[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
     }
   }
+  // The vector body converts pairs with the hardware's round-to-nearest-even instruction
+  // (v_cvt_pk_bf16_f32); the scalar path (narrow1) spells the same rounding with integer
+  // arithmetic.  A NaN comes out as a quiet NaN either way; which one is unspecified (the
+  // host's scalar conversion gives 0x7fc0, its vectorised one 0xffff).
   __device__ static inline u32x4 narrow(const float (&v)[kVec]) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
     u32x4 raw;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      raw[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 pair = {v[2 * i], v[2 * i + 1]};
+      raw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+    }
     return raw;
   }
   __device__ static inline float widen1(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
@@ -257,8 +265,14 @@ struct FlatLocator {
 //   NCOL            number of pointer columns
 //   rmask()/wmask() which columns are loaded / stored (uniform)
 //   apply(v)        per-element arithmetic on v[NCOL] (fp32)
+//   kHasFast, fast(), apply_fast(v)
+//                   optionally, the same arithmetic for the common configuration with
+//                   the uniform decisions (who participates, which SGD terms exist,
+//                   whether the divisor is a power of two) taken once per workgroup
+//                   instead of once per element; fast() is uniform and apply_fast
+//                   returns bit for bit what apply returns whenever fast() holds
 // ---------------------------------------------------------------------------
-template <class E, class Op, int U, bool NT, bool CHECK>
+template <class E, class Op, int U, bool NT, bool CHECK, bool FAST = false>
 __device__ inline void stream_block(char* const (&ptr)[Op::NCOL], const Op& op, uint32_t v0,
                                     uint32_t nvec, uint32_t rmask, uint32_t wmask) {
   constexpr int NCOL = Op::NCOL;
@@ -290,7 +304,10 @@ __device__ inline void stream_block(char* const (&ptr)[Op::NCOL], const Op& op, 
       float v[NCOL];
 #pragma unroll
       for (int c = 0; c < NCOL; ++c) v[c] = lanes[c][i];
-      op.apply(v);
+      if constexpr (FAST)
+        op.apply_fast(v);
+      else
+        op.apply(v);
 #pragma unroll
       for (int c = 0; c < NCOL; ++c) lanes[c][i] = v[c];
     }
@@ -345,6 +362,12 @@ __global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_
   if (w.n == 0) return;
   if (w.vec) {
     if (w.n == kSlab) {
+      if constexpr (Op::kHasFast) {
+        if (op.fast()) {
+          stream_block<E, Op, U, NT, false, true>(ptr, op, 0, kSlab / V, rmask, wmask);
+          return;
+        }
+      }
       stream_block<E, Op, U, NT, false>(ptr, op, 0, kSlab / V, rmask, wmask);
     } else {
       const uint32_t nvec = w.n / V;
@@ -362,6 +385,18 @@ __global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_
 // re-associate them; the fused multiply-adds are the ones torch's own add(alpha)
 // kernels perform.
 // ---------------------------------------------------------------------------
+// num_participants as the kernels see it.  Dividing by a power of two and multiplying by
+// its (exact) reciprocal are the same real number rounded once, so the product replaces
+// the IEEE division bit for bit: inv is that reciprocal, or 0 when n is no power of two.
+struct Divisor {
+  float n, inv;
+};
+
+Divisor make_divisor(uint32_t num_participants) {
+  const bool pow2 = num_participants && !(num_participants & (num_participants - 1u));
+  return Divisor{(float)num_participants, pow2 ? 1.0f / (float)num_participants : 0.0f};
+}
+
 template <int NREP>
 __device__ inline float replica_sum(const float* x, uint32_t mask) {
   // sequential in replica order; a non-participant contributes +0
@@ -375,14 +410,25 @@ __device__ inline float replica_sum(const float* x, uint32_t mask) {
 template <int NOUT, int NREP>
 struct ReduceAvgOp {
   static constexpr int NCOL = NOUT + NREP;
+  static constexpr bool kHasFast = NREP > 0;
   uint32_t mask;  // participation bits
-  float n;        // num_participants
+  Divisor d;      // num_participants
   __device__ inline uint32_t rmask() const { return mask << NOUT; }
   __device__ inline uint32_t wmask() const { return (1u << NOUT) - 1u; }
   __device__ inline void apply(float (&v)[NCOL]) const {
     float s = 0.0f;
     if constexpr (NREP > 0) s = replica_sum<NREP>(&v[NOUT], mask);
-    s = __fdiv_rn(s, n);
+    s = __fdiv_rn(s, d.n);
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) v[o] = s;
+  }
+  // everybody participates and the divisor is a power of two
+  __device__ inline bool fast() const { return mask == (1u << NREP) - 1u && d.inv != 0.0f; }
+  __device__ inline void apply_fast(float (&v)[NCOL]) const {
+    float s = v[NOUT];
+#pragma unroll
+    for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, v[NOUT + r]);
+    s = __fmul_rn(s, d.inv);
 #pragma unroll
     for (int o = 0; o < NOUT; ++o) v[o] = s;
   }
@@ -406,6 +452,26 @@ __device__ inline float sgd_update(const SgdCoef& k, float g, float b, float& bu
   return __fmaf_rn(e, k.neg_lr, b);
 }
 
+// the usual outer optimizer: Nesterov momentum, no weight decay, not the first step
+__device__ inline bool sgd_is_common(const SgdCoef& k) {
+  return k.weight_decay == 0.0f && k.momentum != 0.0f && !k.first_step && k.nesterov;
+}
+
+__device__ inline float sgd_update_common(const SgdCoef& k, float g, float b, float& buf) {
+  const float nb = __fmaf_rn(g, k.one_minus_dampening, __fmul_rn(buf, k.momentum));
+  buf = nb;
+  return __fmaf_rn(__fmaf_rn(nb, k.momentum, g), k.neg_lr, b);
+}
+
+// everybody participates and the divisor is a power of two
+template <int NREP>
+__device__ inline float pseudograd_avg_all(const float* x, float b, float inv) {
+  float s = __fsub_rn(x[0], b);
+#pragma unroll
+  for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, __fsub_rn(x[r], b));
+  return __fmul_rn(s, inv);
+}
+
 template <int NREP>
 __device__ inline float pseudograd_avg(const float* x, float b, uint32_t mask, float n) {
   // each replica subtracts the (shared) backup first, then the differences are summed
@@ -419,8 +485,9 @@ __device__ inline float pseudograd_avg(const float* x, float b, uint32_t mask, f
 template <int NREP>
 struct DilocoFusedOp {
   static constexpr int NCOL = 3 + NREP;
+  static constexpr bool kHasFast = NREP > 0;
   uint32_t mask;
-  float n;
+  Divisor d;
   SgdCoef k;
   __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
   __device__ inline uint32_t rmask() const {
@@ -428,8 +495,17 @@ struct DilocoFusedOp {
   }
   __device__ inline uint32_t wmask() const { return 3u | (uses_buf() ? 4u : 0u); }
   __device__ inline void apply(float (&v)[NCOL]) const {
-    const float g = pseudograd_avg<NREP>(&v[3], v[1], mask, n);
+    const float g = pseudograd_avg<NREP>(&v[3], v[1], mask, d.n);
     const float p = sgd_update(k, g, v[1], v[2]);
+    v[0] = p;
+    v[1] = p;
+  }
+  __device__ inline bool fast() const {
+    return mask == (1u << NREP) - 1u && d.inv != 0.0f && sgd_is_common(k);
+  }
+  __device__ inline void apply_fast(float (&v)[NCOL]) const {
+    const float g = pseudograd_avg_all<NREP>(&v[3], v[1], d.inv);
+    const float p = sgd_update_common(k, g, v[1], v[2]);
     v[0] = p;
     v[1] = p;
   }
@@ -439,13 +515,19 @@ struct DilocoFusedOp {
 template <int NREP>
 struct PseudogradOp {
   static constexpr int NCOL = 3 + NREP;
+  static constexpr bool kHasFast = NREP > 0;
   uint32_t mask;
-  float n;
+  Divisor d;
   uint32_t restore_p;
   __device__ inline uint32_t rmask() const { return (mask << 3) | 4u; }
   __device__ inline uint32_t wmask() const { return 1u | (restore_p ? 2u : 0u); }
   __device__ inline void apply(float (&v)[NCOL]) const {
-    v[0] = pseudograd_avg<NREP>(&v[3], v[2], mask, n);
+    v[0] = pseudograd_avg<NREP>(&v[3], v[2], mask, d.n);
+    v[1] = v[2];
+  }
+  __device__ inline bool fast() const { return mask == (1u << NREP) - 1u && d.inv != 0.0f; }
+  __device__ inline void apply_fast(float (&v)[NCOL]) const {
+    v[0] = pseudograd_avg_all<NREP>(&v[3], v[2], d.inv);
     v[1] = v[2];
   }
 };
@@ -453,6 +535,7 @@ struct PseudogradOp {
 // columns: [p, b, buf, g]
 struct OuterSgdOp {
   static constexpr int NCOL = 4;
+  static constexpr bool kHasFast = true;
   SgdCoef k;
   __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
   __device__ inline uint32_t rmask() const {
@@ -464,6 +547,12 @@ struct OuterSgdOp {
     v[0] = p;
     v[1] = p;
   }
+  __device__ inline bool fast() const { return sgd_is_common(k); }
+  __device__ inline void apply_fast(float (&v)[NCOL]) const {
+    const float p = sgd_update_common(k, v[3], v[1], v[2]);
+    v[0] = p;
+    v[1] = p;
+  }
 };
 
 // columns: [a, scratch]; a is read and written back unchanged, scratch receives a
@@ -472,6 +561,7 @@ struct OuterSgdOp {
 // something the compiler removes, and the probe exists to be timed.
 struct ProbeOp {
   static constexpr int NCOL = 2;
+  static constexpr bool kHasFast = false;
   uint32_t key;
   __device__ inline uint32_t rmask() const { return 1u; }
   __device__ inline uint32_t wmask() const { return 3u; }
@@ -816,7 +906,7 @@ int diloco_outer(const char* what, const tft_mt_table* table, uint32_t n_replica
 #define TFT_CALL(N)                                                                     \
   do {                                                                                  \
     typedef DilocoFusedOp<N> Op;                                                        \
-    const Op op{participate_mask, (float)num_participants, k};                          \
+    const Op op{participate_mask, make_divisor(num_participants), k};                   \
     TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);         \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
@@ -929,7 +1019,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
 #define TFT_CALL(N)                                                             \
   do {                                                                          \
     typedef ReduceAvgOp<1, N> Op;                                               \
-    const Op op{participate_mask, (float)num_participants};                     \
+    const Op op{participate_mask, make_divisor(num_participants)};              \
     TFT_DISPATCH_DTYPE(rc, launch_flat, Op, dtype, what, a, op, shape, s);      \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
@@ -953,7 +1043,7 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
 #define TFT_CALL2(O, N)                                                               \
   do {                                                                                \
     typedef ReduceAvgOp<O, N> Op;                                                     \
-    const Op op{participate_mask, (float)num_participants};                           \
+    const Op op{participate_mask, make_divisor(num_participants)};                    \
     TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);       \
   } while (0)
 #define TFT_CALL_O1(N) TFT_CALL2(1, N)
@@ -995,7 +1085,7 @@ int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
 #define TFT_CALL(N)                                                                   \
   do {                                                                                \
     typedef PseudogradOp<N> Op;                                                       \
-    const Op op{participate_mask, (float)num_participants, restore_p ? 1u : 0u};      \
+    const Op op{participate_mask, make_divisor(num_participants), restore_p ? 1u : 0u}; \
     TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);       \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)

@@ -145,10 +145,10 @@ class DilocoWorkload:
 
 
 def make_diloco_workload(
-    shapes: Named, n_replicas: int, device: torch.device
+    shapes: Named, n_replicas: int, device: torch.device, dtype: torch.dtype = torch.float32
 ) -> DilocoWorkload:
     """backup ~ N(0, 0.02); replica r = backup + N(0, 1e-3) with seed 1000 + r."""
-    backup = normal_tensors(shapes, 0.02, SEED_BACKUP, device)
+    backup = normal_tensors(shapes, 0.02, SEED_BACKUP, device, dtype)
     replicas = [drifted_replica(backup, 1e-3, SEED_REPLICA + r) for r in range(n_replicas)]
     return DilocoWorkload([n for n, _ in shapes], backup, replicas)
 
