@@ -64,9 +64,13 @@ def parse_args() -> argparse.Namespace:
                          "updated in place), flat_backup / flat_momentum (backup / momentum tensors are "
                          "views of one flat allocation, back to back without padding), misaligned (DiLoCo "
                          "workloads: every tensor re-allocated to start 4 bytes past a 16-byte boundary; moved: "
-                         "the same re-allocation, 16 bytes past, as the aligned control), no_placement "
+                         "the same re-allocation, 16 bytes past, as the aligned control; placed: backup "
+                         "and momentum allocated by the library's bank-group placement), no_placement "
                          "(the library allocates backup / momentum / pseudo-gradients without looking "
                          "at HBM bank groups)")
+    ap.add_argument("--model-copies", type=int, default=1,
+                    help="DiLoCo workloads: the tensor list repeated this many times in one launch "
+                         "(separates the fixed cost of a launch from its streaming rate)")
     ap.add_argument("--storage-dtype", choices=("f32", "bf16"), default="f32",
                     help="DiLoCo workloads: dtype of parameters, backup, momentum and replicas "
                          "(arithmetic is fp32 either way; the named configurations are f32)")
@@ -193,6 +197,8 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         shapes, n_rep = workloads.llama3_8b_shapes(), 2
     else:
         shapes, n_rep = workloads.gpt2_small_shapes(), 4
+    if args.model_copies > 1:
+        shapes = [(f"{k}.{name}", sh) for k in range(args.model_copies) for name, sh in shapes]
     dtype = torch.bfloat16 if args.storage_dtype == "bf16" else torch.float32
     esize = 2 if dtype == torch.bfloat16 else 4
     if args.arena and dtype != torch.float32:
@@ -240,8 +246,18 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
             shifted(ts)
         torch.cuda.empty_cache()
         assert all(t.data_ptr() % 16 == (esize * first) % 16 for t in params + wl.backup + bufs)
+    if "placed" in layout:
+        # backup and momentum are the library's buffers: allocated the way DiLoCo allocates them
+        from torchft_amd import hbm_placement
+
+        placed_b, placed_buf = hbm_placement.model_copies(wl.replicas[0], 2)
+        ops.mt_copy(placed_b, wl.backup)
+        ops.mt_copy(placed_buf, bufs)
+        torch.cuda.synchronize()
+        wl.backup, bufs = placed_b, placed_buf
+        torch.cuda.empty_cache()
     for item in layout:
-        if item in ("misaligned", "moved"):
+        if item in ("misaligned", "moved", "placed"):
             continue
         if item == "alias_p":
             params = wl.replicas[0]
@@ -307,10 +323,11 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
          "allocation": ("every tensor is a contiguous view carved out of one device allocation"
                         if args.arena else "one device allocation per tensor"),
-         "layout": layout})
+         "layout": layout, "model_copies": args.model_copies})
     out["roofline"] = roofline(algo_bytes, kernel_ms,
                                f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<{n_rep}>>",
-                               workload=f"diloco_{which}" if esize == 4 else f"diloco_{which}_bf16")
+                               workload="" if args.model_copies > 1 else
+                               (f"diloco_{which}" if esize == 4 else f"diloco_{which}_bf16"))
     if reseeds[0]:
         out["config"]["state_reseeds_inside_timed_region"] = reseeds[0]
         out["roofline"]["note"] = ("steps that re-seed the state include two extra copy launches in "
