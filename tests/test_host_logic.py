@@ -773,6 +773,21 @@ def test_ddp():
     assert call_count >= 1
 
 
+def test_dummy_process_group_under_torch_ddp():
+    """torchft/process_group_test.py:294-298: torch's own DDP wrapper accepts the dummy
+    process group (parameter verification and the initial broadcast go through it)."""
+    from torchft_amd import ProcessGroupDummy
+
+    pg = ProcessGroupDummy(0, 1)
+    m = torch.nn.parallel.DistributedDataParallel(nn.Linear(3, 4), process_group=pg)
+    m(torch.rand(2, 3)).sum().backward()
+    assert all(p.grad is not None for p in m.parameters())
+    assert pg.size() == 1 and pg.getBackendName() == "torchft-dummy"
+    assert pg.configure_count == 0
+    pg.configure("store", 0, 1)
+    assert pg.configure_count == 1
+
+
 def test_ddp_buckets_follow_the_reducer_rule():
     sizes = [p * 4 for p in (2_097_152, 2_048, 4_194_304, 2_048, 20_480, 10)]
     assert compute_bucket_assignment(sizes) == [[1, 2, 3, 4, 5], [0]]

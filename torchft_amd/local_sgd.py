@@ -160,9 +160,9 @@ class LocalSGD:
             and (backup_device is None or torch.device(backup_device) == named[0][1].device)
         ):
             # backup in HBM next to the parameters.  On MI355X concurrent write streams slow
-            # each other down inside one HBM bank group, so large models get per-tensor
-            # buffers in a group their parameter does not occupy (and the outer momentum,
-            # if there will be one, in the third group); otherwise views into one
+            # each other down inside one HBM bank group, so models of some size get
+            # per-tensor buffers (the backup and, if there will be one, the outer momentum)
+            # in a group their parameter does not occupy; otherwise views into one
             # allocation per dtype
             datas = [p.data for _, p in named]
             placed = hbm_placement.allocate_apart(datas, self._placed_copies())
@@ -473,7 +473,15 @@ class DiLoCo(LocalSGD):
                 return [self._placed_momentum[i] for i in idx]
             key = "momentum/" + ",".join(map(str, idx[:4])) + f"/{len(idx)}"
             return self._flat_like(key, [live[i].data for i in idx])[1]
-        return [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
+        bufs = [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
+        placed = self._placed_momentum
+        if placed is not None and len(idx) == len(live) and all(
+            b.data_ptr() != placed[i].data_ptr() for b, i in zip(bufs, idx)
+        ):
+            # the optimizer state was replaced (a load_state_dict after healing): the buffers
+            # allocated for it at construction are not in use any more
+            self._placed_momentum = None
+        return bufs
 
     def _attach_momentum(self, idx: Sequence[int], bufs: Sequence[torch.Tensor]) -> None:
         """After a committed first step the buffers become optimizer state, exactly where
