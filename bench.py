@@ -39,7 +39,8 @@ LR, MOMENTUM = 0.7, 0.9
 HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8B DiLoCo"
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
              "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
-             "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b"]
+             "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b",
+             "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -662,7 +663,7 @@ def bench_host_backup(args) -> Dict[str, object]:
     return out
 
 
-def bench_ddp_buckets(args) -> Dict[str, object]:
+def bench_ddp_buckets(args, form: str = "hook_order") -> Dict[str, object]:
     from torchft_amd import GradBucketAverager, workloads
 
     dev = torch.device("cuda", 0)
@@ -671,8 +672,20 @@ def bench_ddp_buckets(args) -> Dict[str, object]:
     averager = GradBucketAverager(grads[0], grads)  # in place on replica 0, like a DDP bucket
     mask, n = 0b0111, 3  # replica 3 is a spare: zeroed, never read
 
-    def step() -> None:
-        averager.average_all(mask, n)
+    if form == "hook_order":
+        def step() -> None:
+            averager.average_all(mask, n, streams=1)  # what 162 hook calls in a row do
+        how, launches = "one launch per bucket, in hook order on one stream", len(averager.buckets)
+    elif form == "two_streams":
+        def step() -> None:
+            averager.average_all(mask, n, streams=2)  # the library's default for average_all
+        how = ("one launch per bucket in hook order, alternating between two side streams; a step is "
+               "timed from the fork to the join on the current stream")
+        launches = len(averager.buckets)
+    else:
+        def step() -> None:
+            averager.average_whole_model(mask, n)
+        how, launches = "all buckets in one launch", 1
 
     wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(step)
     n_elems = sum(g.numel() for g in grads[0])
@@ -680,12 +693,15 @@ def bench_ddp_buckets(args) -> Dict[str, object]:
                     n_elems / (wall_ms * 1e-3), "elements/s", wall_ms, "bf16 storage, f32 accumulate",
                     {"workload": f"bf16 gradients of Llama-3-8B ({len(shapes)} tensors, {n_elems} "
                                  f"elements) in {len(averager.buckets)} buckets by torch's 1 MiB / 25 MiB "
-                                 "rule, 4 contributions with 3 participating, one launch per bucket "
+                                 f"rule, 4 contributions with 3 participating, {how}, "
                                  "over per-parameter views (no flatten / unflatten passes)",
                      "n_buckets": len(averager.buckets), "n_elements": n_elems})
     out["roofline"] = roofline(n_elems * 2 * (3 + 1), kernel_ms,
-                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", len(averager.buckets),
-                               workload="ddp_buckets_llama3_8b")
+                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>>", launches,
+                               workload="ddp_buckets_llama3_8b" if form == "hook_order" else "")
+    if form == "two_streams":
+        out["roofline"]["note"] = ("launches on the two streams overlap: kernel_ms_per_step is the span from "
+                                   "fork to join, not the sum of the kernels' durations")
     if not args.no_cpu_baseline:
         from oracle import replica_sync as O
 
@@ -874,6 +890,10 @@ def main() -> int:
         out = bench_diloco(args, "gpt2_small")
     elif args.workload == "ddp_buckets_llama3_8b":
         out = bench_ddp_buckets(args)
+    elif args.workload == "ddp_buckets_llama3_8b_two_streams":
+        out = bench_ddp_buckets(args, "two_streams")
+    elif args.workload == "ddp_whole_model_llama3_8b":
+        out = bench_ddp_buckets(args, "one_launch")
     elif args.workload == "checkpoint_llama3_8b":
         out = bench_checkpoint(args)
     elif args.workload == "diloco_llama3_8b_api":

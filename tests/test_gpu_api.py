@@ -461,6 +461,35 @@ def test_grad_bucket_averager(device, dtype):
         assert_bits_equal(out[i], want[i])
 
 
+@pytest.mark.parametrize("streams", [1, 2, 3])
+def test_grad_bucket_averager_all_buckets_over_side_streams(device, streams):
+    """``average_all`` alternates its launches between side streams: it must see what the
+    current stream wrote just before the call, and what it writes must be visible to the
+    current stream right after it (no synchronisation by the caller)."""
+    shapes = workloads.gpt2_small_shapes()[:60]
+    grads = workloads.make_grad_replicas(shapes, 3, torch.device("cpu"), torch.bfloat16)
+    numels = [g.numel() for g in grads[0]]
+    buckets = O.bucket_assignment(numels, 2)
+    assert len(buckets) > 3
+    doubled = [[(t.float() * 2).to(torch.bfloat16) for t in rep] for rep in grads]
+    want = O.ddp_bucket_average(doubled, [True, True, True], 3, buckets, torch.float32)
+    dev = [[t.to(device) for t in rep] for rep in grads]
+    out = [torch.empty_like(t) for t in dev[0]]
+    avg = GradBucketAverager(out, dev)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):  # a non-default current stream, to make ordering matter
+        for rep in dev:
+            torch._foreach_mul_(rep, 2.0)  # producer on the current stream
+        avg.average_all(streams=streams)
+        sums = [t.float().sum() for t in out]  # consumer on the current stream
+    side.synchronize()
+    for i, (name, _) in enumerate(shapes):
+        assert_bits_equal(out[i], want[i], name)
+        assert float(sums[i]) == float(want[i].float().sum().to(torch.float32)) or torch.isclose(
+            sums[i].cpu(), want[i].float().sum(), rtol=1e-3, atol=1e-3)
+
+
 def test_flatten_unflatten_are_byte_exact(device):
     """Bucket flatten / unflatten as explicit copies (what the Reducer does around the hook):
     offsets are running element counts with no padding."""
