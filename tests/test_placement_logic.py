@@ -1,0 +1,168 @@
+"""The bank-group search of torchft_amd.hbm_placement as host logic, without a GPU: device
+memory is one host arena whose byte ranges are assigned to three fake bank groups, and the
+probe is a function of the two buffers' groups (plus noise), as the real timings are."""
+
+import random
+
+import pytest
+import torch
+
+from torchft_amd import hbm_placement as H
+
+MiB = 1 << 20
+
+
+class FakeDevice:
+    """A bump allocator over one arena.  Like the GPU driver it hands memory out in address
+    order; every ``group_bytes`` the next bank group starts."""
+
+    def __init__(self, total=96 * MiB, group_bytes=24 * MiB, n_groups=3, noise=0.0, seed=0):
+        self.arena = torch.zeros(total, dtype=torch.uint8)
+        self.base = self.arena.data_ptr()
+        self.total, self.group_bytes, self.n_groups = total, group_bytes, n_groups
+        self.cursor = 0
+        self.noise, self.rng = noise, random.Random(seed)
+        self.released = 0
+        self.probes = 0
+
+    def allocate(self, nbytes: int) -> torch.Tensor:
+        start = -(-self.cursor // 256) * 256
+        if start + nbytes > self.total:
+            raise RuntimeError("fake device out of memory")
+        self.cursor = start + nbytes
+        return self.arena[start:start + nbytes]
+
+    def free_memory(self) -> int:
+        return self.total - self.cursor
+
+    def release(self) -> None:
+        self.released += 1
+
+    def group_at(self, t: torch.Tensor, last: bool = False) -> int:
+        off = t.data_ptr() - self.base + (t.numel() * t.element_size() - 1 if last else 0)
+        return (off // self.group_bytes) % self.n_groups
+
+    def probe_ms(self, a, b, nbytes=None, repeats=3):
+        self.probes += 1
+        n = min(a.numel() * a.element_size(), b.numel() * b.element_size(), nbytes or H.PROBE_BYTES)
+        same = self.group_at(a) == self.group_at(b)
+        ms = (1.0 if same else 0.83) * n / MiB
+        return ms * (1.0 + self.rng.uniform(-self.noise, self.noise)) + 0.0
+
+
+@pytest.fixture
+def small_constants(monkeypatch):
+    monkeypatch.setattr(H, "PROBE_BYTES", 256 << 10)
+    monkeypatch.setattr(H, "MIN_PROBE_BYTES", 64 << 10)
+    monkeypatch.setattr(H, "BLOCK_BYTES", 1 * MiB)
+    monkeypatch.setattr(H, "BLOCK_GRANULE", 1 * MiB)
+    monkeypatch.setattr(H, "NO_STRUCTURE_BYTES", 40 * MiB)
+
+
+def make_pool(dev: FakeDevice, monkeypatch) -> H.GroupedPool:
+    monkeypatch.setattr(H, "probe_ms", dev.probe_ms)
+    pool = H.GroupedPool(torch.device("cpu"), allocate=dev.allocate, free_memory=dev.free_memory,
+                         release=dev.release)
+    pool.keep_free = 2 * MiB
+    return pool
+
+
+def model_on(dev: FakeDevice, sizes):
+    return [dev.allocate(n * 4).view(torch.float32) for n in sizes]
+
+
+@pytest.mark.parametrize("noise", [0.0, 0.015])
+def test_blocks_are_classified_and_buffers_land_in_the_next_group(small_constants, monkeypatch, noise):
+    dev = FakeDevice(noise=noise, seed=3)
+    # a model of 6 MiB at the start of group 0: two probe-sized tensors and small ones
+    like = model_on(dev, [MiB // 2, 1000, MiB // 2, 10, 300_000])
+    pool = make_pool(dev, monkeypatch)
+    sizes = [t.numel() * 4 for t in like]
+    copies = H._allocate_apart(like, sizes, 2, torch.device("cpu"), pool=pool)
+    assert copies is not None and len(copies) == 2
+    assert len(pool.map.anchors) == 3
+    seen = []
+    for copy in copies:
+        for t, ref in zip(copy, like):
+            assert t.shape == ref.shape and t.dtype == ref.dtype
+            assert (t.data_ptr() - dev.base) % 256 == 0
+            # entirely inside the group after the model's
+            assert dev.group_at(t) == dev.group_at(t, last=True) == (dev.group_at(ref) + 1) % 3
+            seen.append((t.data_ptr(), t.data_ptr() + t.numel() * 4))
+    seen.sort()
+    assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(seen, seen[1:])), "buffers overlap"
+    assert dev.released >= 1  # what the search held and did not use went back
+    assert all(b.used > 0 for b in pool.blocks)
+
+
+def test_a_model_across_two_groups_gets_each_tensor_its_own_neighbour(small_constants, monkeypatch):
+    dev = FakeDevice(group_bytes=8 * MiB, total=64 * MiB)
+    like = model_on(dev, [MiB] * 3)  # 4 MiB each: tensors 0, 1 in group 0, tensor 2 in group 1
+    assert [dev.group_at(t) for t in like] == [0, 0, 1]
+    pool = make_pool(dev, monkeypatch)
+    copies = H._allocate_apart(like, [t.numel() * 4 for t in like], 1, torch.device("cpu"), pool=pool)
+    got = [dev.group_at(t) for t in copies[0]]
+    # group indices of the pool are in order of discovery, which here is the device's order
+    assert got == [1, 1, 2]
+
+
+def test_a_block_across_a_boundary_is_held_but_never_used(small_constants, monkeypatch):
+    dev = FakeDevice(group_bytes=8 * MiB + 512 * 1024, total=64 * MiB)  # boundaries inside blocks
+    like = model_on(dev, [MiB // 2])
+    pool = make_pool(dev, monkeypatch)
+    copies = H._allocate_apart(like, [like[0].numel() * 4], 2, torch.device("cpu"), pool=pool)
+    assert copies is not None
+    for copy in copies:
+        t = copy[0]
+        assert dev.group_at(t) == dev.group_at(t, last=True) != dev.group_at(like[0])
+    for b in pool.blocks:
+        assert dev.group_at(b.storage) == dev.group_at(b.storage, last=True)
+
+
+def test_a_device_without_groups_is_left_alone(small_constants, monkeypatch):
+    dev = FakeDevice(n_groups=1, total=64 * MiB)
+    like = model_on(dev, [MiB // 2])
+    pool = make_pool(dev, monkeypatch)
+    assert H._allocate_apart(like, [like[0].numel() * 4], 1, torch.device("cpu"), pool=pool) is None
+    assert not pool.structured and len(pool.map.anchors) == 1
+    assert pool.blocks == [] and dev.released >= 1
+
+
+def test_running_out_of_memory_falls_back_to_the_other_groups(small_constants, monkeypatch):
+    # the device ends inside group 1: what does not fit there goes to group 0 (there is no
+    # group 2 to be found), and what fits nowhere in the pool is allocated plainly
+    dev = FakeDevice(group_bytes=8 * MiB, total=15 * MiB)
+    like = model_on(dev, [MiB // 2, MiB // 2, MiB // 2])  # 6 MiB in group 0
+    pool = make_pool(dev, monkeypatch)
+    pool.keep_free = 0
+    sizes = [t.numel() * 4 for t in like]
+    copies = H._allocate_apart(like, sizes, 1, torch.device("cpu"), pool=pool)
+    assert copies is not None and len(pool.map.anchors) == 2
+    groups = sorted(dev.group_at(t) for t in copies[0])
+    assert groups.count(1) >= 2  # group 1 first, for as long as it has room
+    for t, ref in zip(copies[0], like):
+        assert t.shape == ref.shape and dev.group_at(t) == dev.group_at(t, last=True)
+
+
+def test_small_tensors_take_the_group_of_their_nearest_probed_neighbour(small_constants, monkeypatch):
+    dev = FakeDevice(group_bytes=8 * MiB, total=64 * MiB)
+    a = dev.allocate(512 << 10).view(torch.float32)       # group 0, probed
+    small0 = dev.allocate(1000).view(torch.uint8)           # next to it
+    dev.cursor = 9 * MiB
+    b = dev.allocate(512 << 10).view(torch.float32)       # group 1, probed
+    small1 = dev.allocate(1000).view(torch.uint8)
+    pool = make_pool(dev, monkeypatch)
+    pool.grow_until(lambda pl: len(pl.map.anchors) >= 3)
+    groups = H.groups_of_tensors(pool, [a, small0, b, small1])
+    assert groups[0] == groups[1] and groups[2] == groups[3] and groups[0] != groups[2]
+
+
+def test_allocate_apart_declines_what_it_cannot_help(monkeypatch):
+    cpu = [torch.zeros(10)]
+    assert H.allocate_apart(cpu, 1) is None            # not on a GPU
+    assert H.allocate_apart([], 1) is None
+    assert H.allocate_apart(cpu, 3) is None            # one or two copies only
+    monkeypatch.setenv("TORCHFT_AMD_HBM_PLACEMENT", "0")
+    assert not H.enabled()
+    copies = H.model_copies(cpu, 2)                    # plain allocations instead
+    assert len(copies) == 2 and copies[0][0].shape == cpu[0].shape

@@ -40,7 +40,7 @@ import ctypes
 import logging
 import os
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -53,11 +53,13 @@ N_GROUPS = 3
 PROBE_BYTES = 512 << 20      # per buffer and probe: long enough to time reliably (0.3 ms), short enough to be free
 MIN_PROBE_BYTES = 128 << 20  # tensors below this are not probed (they take their neighbour's group)
 BLOCK_BYTES = 2 << 30        # device memory is taken from torch in blocks of this size
+BLOCK_GRANULE = 1 << 30      # ... or of the largest tensor's size rounded up to this, if that is more
 # probe time / time of a same-group pair: 0.97-1.05 measured inside one group, 0.83-0.85
 # across two (probes of 128 MiB and more)
 SAME_GROUP_RATIO = 0.92
 AMBIGUOUS_BAND = 0.03        # a ratio this close to the threshold is measured again
 RELATIVE_CONTRAST = 1.06     # own-group probe time / next longest, with all three anchors known
+NO_STRUCTURE_BYTES = 110 << 30  # this much memory in ONE group: the device has no such groups
 MIN_MODEL_BYTES = 256 << 20  # smaller models are left alone (a GPT-2-small of 0.5 GB still gains 1-2 %)
 ALIGN = 256
 
@@ -138,7 +140,7 @@ class GroupMap:
         An unclear measurement is repeated with more launches."""
         size = _as_bytes(t).numel()
         n = min(size, PROBE_BYTES if nbytes is None else nbytes) // 16 * 16
-        if n < MIN_PROBE_BYTES:
+        if n < MIN_PROBE_BYTES or not self.anchors:
             return None
         for repeats in (3, 6, 9):
             times = [probe_ms(t, anchor, n, repeats) for anchor in self.anchors]
@@ -165,12 +167,24 @@ class GroupedPool:
     ``release_unused`` returns the untouched ones.
     """
 
-    def __init__(self, device: torch.device) -> None:
+    def __init__(
+        self,
+        device: torch.device,
+        allocate: Optional[Callable[[int], torch.Tensor]] = None,
+        free_memory: Optional[Callable[[], int]] = None,
+        release: Optional[Callable[[], None]] = None,
+    ) -> None:
         self.device = device
         self.map = GroupMap(device)
         self.blocks: List[_Block] = []
         self._straddling: List[torch.Tensor] = []  # blocks across a group boundary: held, unused
         self.structured = True  # False once the timings show no group structure
+        # where blocks come from and go back to (replaceable: the search logic is host code
+        # and is tested without a GPU)
+        self._allocate = allocate or (lambda n: torch.empty(n, dtype=torch.uint8, device=device))
+        self._free_memory = free_memory or (lambda: torch.cuda.mem_get_info(device)[0])
+        self._release = release or torch.cuda.empty_cache
+        self.keep_free = 6 << 30  # device memory the search never touches
 
     # -- discovery ---------------------------------------------------------------
     def _classify_block(self, storage: torch.Tensor) -> Optional[int]:
@@ -204,24 +218,25 @@ class GroupedPool:
     def free_bytes(self, group: int) -> int:
         return sum(b.free() for b in self.blocks if b.group == group)
 
-    def grow_until(self, satisfied, keep_free: int = 6 << 30, block_bytes: int = BLOCK_BYTES) -> bool:
+    def grow_until(self, satisfied, keep_free: Optional[int] = None, block_bytes: Optional[int] = None) -> bool:
         """Takes blocks from the device, one at a time, until ``satisfied(self)`` holds; False if
         the device ran out first.  Every block that lies in one group is kept as a candidate
         (the driver hands physical memory out in address order, so the way to the next group
         leads through the rest of the current one: what is not wanted must be held, not
         returned, until the search is over - ``release_unused`` gives it back)."""
+        keep_free = self.keep_free if keep_free is None else keep_free
+        block_bytes = BLOCK_BYTES if block_bytes is None else block_bytes
         while not satisfied(self):
-            free, _ = torch.cuda.mem_get_info(self.device)
-            if free < keep_free + block_bytes:
+            if self._free_memory() < keep_free + block_bytes:
                 logger.info("hbm placement: device memory ran out before the search was satisfied")
                 return False
-            storage = torch.empty(block_bytes, dtype=torch.uint8, device=self.device)
+            storage = self._allocate(block_bytes)
             g = self._classify_block(storage)
             if g is None:
                 self._straddling.append(storage)
             else:
                 self.blocks.append(_Block(storage, g))
-            if len(self.map.anchors) == 1 and len(self.blocks) * block_bytes > (110 << 30):
+            if len(self.map.anchors) == 1 and len(self.blocks) * block_bytes > NO_STRUCTURE_BYTES:
                 # more than a whole group's worth of memory and still one group: this
                 # device shows no group structure
                 self.structured = False
@@ -251,7 +266,7 @@ class GroupedPool:
         """Gives every block nothing was taken from back to the device."""
         self.blocks = [b for b in self.blocks if b.used > 0]
         self._straddling = []
-        torch.cuda.empty_cache()
+        self._release()
 
 
 def groups_of_tensors(pool: GroupedPool, tensors: Sequence[torch.Tensor]) -> List[Optional[int]]:
@@ -299,12 +314,14 @@ def allocate_apart(
 
 
 def _allocate_apart(
-    like: Sequence[torch.Tensor], sizes: List[int], n_copies: int, device: torch.device
+    like: Sequence[torch.Tensor], sizes: List[int], n_copies: int, device: torch.device,
+    pool: Optional[GroupedPool] = None,
 ) -> Optional[List[List[torch.Tensor]]]:
-    torch.cuda.synchronize(device)
-    pool = GroupedPool(device)
+    if pool is None:
+        torch.cuda.synchronize(device)
+        pool = GroupedPool(device)
     largest = max(sizes)
-    block = max(BLOCK_BYTES, -(-largest // (1 << 30)) * (1 << 30))
+    block = max(BLOCK_BYTES, -(-largest // BLOCK_GRANULE) * BLOCK_GRANULE)
     # first: reach all groups, so that there is an anchor to compare the model with in each
     pool.grow_until(lambda pl: len(pl.map.anchors) >= N_GROUPS, block_bytes=block)
     if not pool.structured or len(pool.map.anchors) < 2:
@@ -342,7 +359,7 @@ def _allocate_apart(
     pool.release_unused()
     for (i, k), raw in list(placed.items()):
         if raw is None:
-            raw = torch.empty(max(sizes[i], 1), dtype=torch.uint8, device=device)[: sizes[i]]
+            raw = pool._allocate(max(sizes[i], 1))[: sizes[i]]
         placed[(i, k)] = raw.view(like[i].dtype).view(like[i].shape)
     for k in range(n_copies):
         copies[k] = [placed[(i, k)] for i in range(len(like))]
