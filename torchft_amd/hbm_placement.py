@@ -5,19 +5,19 @@ group is a contiguous range of physical memory.  Streams that are WRITTEN
 concurrently slow each other down when they lie in the same group: a pair of
 in-place (read + write) streams runs at 5.6 TB/s inside one group against
 6.4 TB/s across two, two pure write streams at 5.8 against 7.1 TB/s, and a
-LocalSGD average whose parameters and backup share a group at 0.70 of the
-8 TB/s peak against 0.82 when they do not.  Read-only streams do not care.
+LocalSGD average whose parameters and backup share a group at 0.79 of the
+8 TB/s peak against 0.85 when they do not.  Read-only streams do not care.
 
 The replica-sync kernels write the live parameters, the backup and the outer
-momentum at the same element offsets at the same time.  Measured over all
+momentum at the same element offsets at the same time.  Measured over the
 assignments of the streams to groups (fused DiLoCo step, parameters updated in
-place): everything in one group 0.69 of peak - which is exactly what a model of
+place): everything in one group 0.77 of peak - which is exactly what a model of
 up to 32 GB gets when its backup and momentum are allocated right behind it -
-against 0.78-0.79 as soon as backup and momentum lie outside the parameters'
-group; the best of those keeps backup and momentum TOGETHER in one other group
-(splitting them over the two remaining groups is 1 % slower).  For the LocalSGD
-average the same move is worth 0.70 -> 0.82.  The parameters are the user's; the
-backup and momentum buffers are allocated here, so this module
+against 0.80 as soon as backup and momentum lie outside the parameters' group;
+keeping them TOGETHER in one other group is as good as or better than splitting
+them over the two remaining groups.  For the LocalSGD average the same move is
+worth 0.79 -> 0.85.  The parameters are the user's; the backup and momentum
+buffers are allocated here, so this module
 
 * finds out which group a piece of device memory lies in.  Virtual addresses
   say nothing about it, and there is no query for it; what tells is time: the
