@@ -64,6 +64,8 @@ _DEADLINES = _Deadlines()
 
 def future_timeout(fut: "Future[T]", timeout: timedelta) -> "Future[T]":
     """A future with the value (or error) of ``fut``, or a ``TimeoutError`` after ``timeout``."""
+    if fut.done():
+        return fut  # nothing left to time (stream-ordered work completes its future at launch)
     timed: Future = Future()
     lock = threading.Lock()
     done = [False]
