@@ -345,9 +345,12 @@ def test_diloco_gpt2_small_four_replicas(device):
 # DDP
 # ---------------------------------------------------------------------------
 
-def test_ddp_comm_hook_on_gpu(device):
+@pytest.mark.parametrize("bucket_views", [False, True])
+def test_ddp_comm_hook_on_gpu(device, bucket_views):
     """torch's Reducer flattens, the hook's Manager.allreduce averages the flat bucket with
-    one kernel, the Reducer unflattens: gradients equal the checker's bucket average."""
+    one kernel, the Reducer unflattens: gradients equal the checker's bucket average.  With
+    ``gradient_as_bucket_view=True`` the gradients are views of the bucket, so the Reducer's
+    two copies disappear and the kernel's pass is the only one."""
     torch.manual_seed(0)
     model = MLP().to(device)
     captured = {}
@@ -360,12 +363,15 @@ def test_ddp_comm_hook_on_gpu(device):
 
     pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
     manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, quorum_client=StaticQuorum(0, 2))
-    ddp = DistributedDataParallel(manager, model)
+    ddp = DistributedDataParallel(manager, model, gradient_as_bucket_view=bucket_views)
     manager.start_quorum()
     ddp(torch.randn(4, 1024, device=device)).square().mean().backward()
     torch.cuda.synchronize()
     assert manager.should_commit()
     assert len(captured) == 2  # two buckets for this model (4 218 890 and 2 097 152 elements)
+    if bucket_views:  # every gradient lies inside one of the two flat buffers the hook saw
+        spans = [(ptr, ptr + 4 * v[0].numel()) for ptr, v in captured.items()]
+        assert all(any(lo <= p.grad.data_ptr() < hi for lo, hi in spans) for p in model.parameters())
     params = list(model.parameters())
     numels = [p.numel() for p in params]
     buckets = O.bucket_assignment(numels, 4)
