@@ -46,7 +46,8 @@ def reduce_avg_table(outs, replicas):
     return FakeTable()
 
 
-def mt_reduce_avg(outs, replicas, participate_mask=None, num_participants=None, table=None):
+def mt_reduce_avg(outs, replicas, participate_mask=None, num_participants=None, table=None,
+                  table_is_current=False):
     calls.append("mt_reduce_avg")
     n = len(replicas)
     mask = real_ops.full_mask(n) if participate_mask is None else participate_mask
@@ -101,7 +102,7 @@ def diloco_outer_table(params, backups, bufs, replicas, table=None):
 
 
 def mt_diloco_outer(params, backups, bufs, replicas, sgd, first_step, participate_mask=None,
-                    num_participants=None, table=None):
+                    num_participants=None, table=None, table_is_current=False):
     calls.append("mt_diloco_outer")
     n = len(replicas)
     mask = real_ops.full_mask(n) if participate_mask is None else participate_mask

@@ -349,7 +349,7 @@ class LocalSGD:
             assert launches, "a replica that failed to prepare cannot have voted to commit"
             for key, outs, reps, mask, table in launches:
                 self._tables[key] = ops.mt_reduce_avg(
-                    outs, reps, mask, manager.num_participants(), table=table
+                    outs, reps, mask, manager.num_participants(), table=table, table_is_current=True
                 )
         else:
             self._restore_parameters()
@@ -622,7 +622,7 @@ class DiLoCo(LocalSGD):
             for key, idx, cols, sgd, first, mask, table in launches:
                 self._tables[key] = ops.mt_diloco_outer(
                     cols["params"], cols["backups"], cols["bufs"], cols["replicas"], sgd, first,
-                    mask, manager.num_participants(), table=table,
+                    mask, manager.num_participants(), table=table, table_is_current=True,
                 )
                 if first and cols["bufs"] is not None:
                     self._attach_momentum(idx, cols["bufs"])

@@ -10,6 +10,8 @@ host-to-device traffic.
 from __future__ import annotations
 
 import ctypes
+import itertools
+import operator
 from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -22,6 +24,11 @@ _DTYPE_CODES = {
     torch.bfloat16: _native.TFT_BF16,
     torch.float16: _native.TFT_F16,
 }
+
+
+_DATA_PTR = torch.Tensor.data_ptr
+_NUMEL = torch.Tensor.numel
+_DTYPE = operator.attrgetter("dtype")
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -190,7 +197,15 @@ class TensorTable:
 
     @staticmethod
     def make_key(columns: Sequence[Sequence[torch.Tensor]]) -> Tuple:
-        return tuple((x.data_ptr(), x.numel(), x.dtype) for col in columns for x in col)
+        """Identity of the tensors a table describes: address, size and dtype of every one
+        (checked on every launch, so built with C-level maps rather than a Python loop)."""
+        flat = list(itertools.chain.from_iterable(columns))
+        return (
+            tuple(map(_DATA_PTR, flat)),
+            tuple(map(_NUMEL, flat)),
+            tuple(map(_DTYPE, flat)),
+            tuple(map(len, columns)),
+        )
 
     def matches(self, columns: Sequence[Sequence[torch.Tensor]]) -> bool:
         return self.key == self.make_key(columns)

@@ -119,13 +119,16 @@ def mt_reduce_avg(
     participate_mask: Optional[int] = None,
     num_participants: Optional[int] = None,
     table: Optional[TensorTable] = None,
+    table_is_current: bool = False,
 ) -> TensorTable:
-    """outs[j][t] = (sum_r replicas[r][t]) / n for every tensor t, in one launch."""
+    """outs[j][t] = (sum_r replicas[r][t]) / n for every tensor t, in one launch.
+    ``table_is_current``: the caller has just built or matched ``table`` against exactly
+    these tensors, so it is not compared with them again."""
     n = len(replicas)
     mask = full_mask(n) if participate_mask is None else participate_mask
     nump = n if num_participants is None else num_participants
     _check_reduce_args(n, mask, nump)
-    if table is None or not table.matches([*outs, *replicas]):
+    if table is None or not (table_is_current or table.matches([*outs, *replicas])):
         table = reduce_avg_table(outs, replicas)
     _launch(table, "tft_mt_reduce_avg", len(outs), n, mask, nump, table.dtype_code)
     return table
@@ -156,16 +159,20 @@ def mt_diloco_outer(
     participate_mask: Optional[int] = None,
     num_participants: Optional[int] = None,
     table: Optional[TensorTable] = None,
+    table_is_current: bool = False,
 ) -> TensorTable:
     """Fused DiLoCo outer step (pseudo-gradient, average, Nesterov SGD, backup refresh);
-    fp32, or bf16 / fp16 storage with fp32 arithmetic and one rounding on store."""
+    fp32, or bf16 / fp16 storage with fp32 arithmetic and one rounding on store.
+    ``table_is_current``: ``table`` comes from :func:`diloco_outer_table` for exactly these
+    tensors and is not compared with them again."""
     n = len(replicas)
     mask = full_mask(n) if participate_mask is None else participate_mask
     nump = n if num_participants is None else num_participants
     _check_reduce_args(n, mask, nump)
     if sgd.momentum != 0.0 and bufs is None:
         raise ValueError("momentum != 0 needs momentum buffers")
-    table = diloco_outer_table(params, backups, bufs, replicas, table)
+    if table is None or not table_is_current:
+        table = diloco_outer_table(params, backups, bufs, replicas, table)
     _launch(
         table, "tft_mt_diloco_outer", n, mask, nump, table.dtype_code,
         ctypes.byref(sgd.to_struct(first_step)),
