@@ -81,6 +81,34 @@ def test_diloco_llama3_8b_full_size(device):
     assert all(int(torch.count_nonzero(m)) == 0 for m in bufs[:5])
 
 
+def test_diloco_llama3_8b_full_size_bf16_in_place(device):
+    """The same step on bf16 storage (fp32 arithmetic, one rounding per stored value), updated
+    in place on replica 0 as ``DiLoCo.sync()`` runs it: windows of every tensor against the
+    checker, backup == parameters everywhere, and the peer replica untouched."""
+    shapes = workloads.llama3_8b_shapes()
+    wl = workloads.make_diloco_workload(shapes, 2, device, torch.bfloat16)
+    bufs = [torch.zeros_like(t) for t in wl.backup]
+    params = wl.replicas[0]
+    sgd = ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True)
+    gen = torch.Generator().manual_seed(13)
+    spans = [windows(t.numel(), gen) for t in wl.backup]
+    peer_before = [take(t, s) for t, s in zip(wl.replicas[1], spans)]
+    table = None
+    for step in range(2):
+        before_b = [take(t, s) for t, s in zip(wl.backup, spans)]
+        before_m = [take(t, s) for t, s in zip(bufs, spans)] if step else None
+        reps = [[take(t, s) for t, s in zip(rep, spans)] for rep in wl.replicas]
+        table = ops.mt_diloco_outer(params, wl.backup, bufs, wl.replicas, sgd, step == 0, table=table)
+        want = O.diloco_perform_sync(reps, before_b, before_m, [True, True], 2, True,
+                                     lr=0.7, momentum=0.9, nesterov=True, accumulate_dtype=torch.float32)
+        for i, (name, _) in enumerate(shapes):
+            assert_bits_equal(take(params[i], spans[i]), want["params"][i], f"step {step} {name}")
+            assert_bits_equal(take(bufs[i], spans[i]), want["momentum"][i], f"step {step} momentum {name}")
+        assert all(torch.equal(p, b) for p, b in zip(params, wl.backup))
+    for i in range(len(shapes)):
+        assert_bits_equal(take(wl.replicas[1][i], spans[i]), peer_before[i])
+
+
 def test_ddp_buckets_llama3_8b_full_size(device):
     """bf16 gradients of Llama-3-8B, 162 buckets by torch's rule, 4 contributions of which
     3 participate, fp32 accumulation, result written over replica 0's gradients."""
