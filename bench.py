@@ -40,7 +40,7 @@ HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
              "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
              "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b",
-             "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b"]
+             "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b", "localsgd_llama3_8b_api"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -388,6 +388,46 @@ def bench_diloco_api(args) -> Dict[str, object]:
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
     out["roofline"] = roofline(n_params * 7 * esize, kernel_ms,
                                f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<2>>")
+    out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
+    return out
+
+
+def bench_localsgd_api(args) -> Dict[str, object]:
+    """The LocalSGD average driven through the torchft-shaped API: ``LocalSGD.sync()`` on a
+    module with the 291 Llama-3-8B fp32 parameters, this package's Manager on a local replica
+    group of 2 (quorum, table checks, commit vote, one launch that writes parameters and
+    backup)."""
+    from torch import nn
+
+    from torchft_amd import LocalSGD, Manager, ProcessGroupLocalReplicas, StaticQuorum, workloads
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+
+    class Bag(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList(
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev)])
+
+    model = Bag()
+    peer = workloads.drifted_replica([p.data for p in model.parameters()], 1e-3, 1001)
+    index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = torch.optim.SGD(model.parameters(), lr=0.1)
+    n_params = sum(p.numel() for p in model.parameters())
+    with LocalSGD(manager, model, inner, sync_every=10 ** 9) as local_sgd:
+        wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(local_sgd.sync)
+    manager.shutdown(wait=False)
+    out = base_line(args, "LocalSGD sync params/sec, Llama-3-8B (through LocalSGD.sync())",
+                    n_params / (wall_ms * 1e-3), "params/s", wall_ms, "f32",
+                    {"workload": "LocalSGD.sync() on a module with the 291 Llama-3-8B fp32 parameters, "
+                                 "Manager + ProcessGroupLocalReplicas(world 2); parameters averaged in "
+                                 "place, backup refreshed by the same launch",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
+    out["roofline"] = roofline(n_params * 16, kernel_ms, "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>")
     out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
     return out
 
@@ -900,6 +940,8 @@ def main() -> int:
         out = bench_diloco_api(args)
     elif args.workload == "diloco_two_phase_llama3_8b":
         out = bench_diloco_two_phase(args)
+    elif args.workload == "localsgd_llama3_8b_api":
+        out = bench_localsgd_api(args)
     elif args.workload == "placement_llama3_8b_slice":
         out = bench_placement(args)
     elif args.workload == "host_backup_llama3_8b":
