@@ -59,11 +59,12 @@ def small_constants(monkeypatch):
     monkeypatch.setattr(H, "NO_STRUCTURE_BYTES", 40 * MiB)
 
 
-def make_pool(dev: FakeDevice, monkeypatch) -> H.GroupedPool:
+def make_pool(dev: FakeDevice, monkeypatch, state=None) -> H.GroupedPool:
     monkeypatch.setattr(H, "probe_ms", dev.probe_ms)
     pool = H.GroupedPool(torch.device("cpu"), allocate=dev.allocate, free_memory=dev.free_memory,
-                         release=dev.release)
+                         release=dev.release, state=state, epoch=lambda: dev.released)
     pool.keep_free = 2 * MiB
+    pool.limit = dev.total  # the allowance has a test of its own
     return pool
 
 
@@ -80,7 +81,9 @@ def test_blocks_are_classified_and_buffers_land_in_the_next_group(small_constant
     sizes = [t.numel() * 4 for t in like]
     copies = H._allocate_apart(like, sizes, 2, torch.device("cpu"), pool=pool)
     assert copies is not None and len(copies) == 2
-    assert len(pool.map.anchors) == 3
+    # the search stops as soon as the group after the model's holds what is needed: the third
+    # group is never visited
+    assert len(pool.map.anchors) == 2
     seen = []
     for copy in copies:
         for t, ref in zip(copy, like):
@@ -92,7 +95,9 @@ def test_blocks_are_classified_and_buffers_land_in_the_next_group(small_constant
     seen.sort()
     assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(seen, seen[1:])), "buffers overlap"
     assert dev.released >= 1  # what the search held and did not use went back
-    assert all(b.used > 0 for b in pool.blocks)
+    # what is left holds tensors, or is one of the two anchors' blocks
+    assert all(b.used > 0 or b in pool.state.anchor_blocks for b in pool.blocks)
+    assert len(pool.state.anchor_blocks) == 2
 
 
 def test_a_model_across_two_groups_gets_each_tensor_its_own_neighbour(small_constants, monkeypatch):
@@ -124,7 +129,8 @@ def test_a_device_without_groups_is_left_alone(small_constants, monkeypatch):
     like = model_on(dev, [MiB // 2])
     pool = make_pool(dev, monkeypatch)
     assert H._allocate_apart(like, [like[0].numel() * 4], 1, torch.device("cpu"), pool=pool) is None
-    assert not pool.structured and len(pool.map.anchors) == 1
+    # nothing is kept on such a device, not even the one reference buffer
+    assert not pool.structured and pool.map.anchors == [] and pool.state.anchor_blocks == []
     assert pool.blocks == [] and dev.released >= 1
 
 
@@ -132,7 +138,7 @@ def test_running_out_of_memory_falls_back_to_the_other_groups(small_constants, m
     # the device ends inside group 1: what does not fit there goes to group 0 (there is no
     # group 2 to be found), and what fits nowhere in the pool is allocated plainly
     dev = FakeDevice(group_bytes=8 * MiB, total=15 * MiB)
-    like = model_on(dev, [MiB // 2, MiB // 2, MiB // 2])  # 6 MiB in group 0
+    like = model_on(dev, [MiB * 3 // 8] * 4)  # 4 x 1.5 MiB = 6 MiB in group 0
     pool = make_pool(dev, monkeypatch)
     pool.keep_free = 0
     sizes = [t.numel() * 4 for t in like]
@@ -166,3 +172,167 @@ def test_allocate_apart_declines_what_it_cannot_help(monkeypatch):
     assert not H.enabled()
     copies = H.model_copies(cpu, 2)                    # plain allocations instead
     assert len(copies) == 2 and copies[0][0].shape == cpu[0].shape
+
+
+# ---------------------------------------------------------------------------
+# What a device's state keeps between searches
+# ---------------------------------------------------------------------------
+
+def search(dev, state, like, n_copies, monkeypatch, limit=None):
+    def factory(st):
+        pool = make_pool(dev, monkeypatch, state=st)
+        if limit is not None:
+            pool.limit = limit
+        factory.pools.append(pool)
+        return pool
+
+    factory.pools = []
+    sizes = [t.numel() * 4 for t in like]
+    copies = H._locked_search(state, like, sizes, n_copies, torch.device("cpu"), make_pool=factory)
+    return copies, factory.pools[-1] if factory.pools else None
+
+
+def test_a_second_search_reuses_the_anchors_of_the_first(small_constants, monkeypatch):
+    dev = FakeDevice(total=160 * MiB, group_bytes=32 * MiB)
+    like = model_on(dev, [MiB // 2, MiB // 2, 1000])
+    state = H.DeviceState(torch.device("cpu"))
+    first, pool1 = search(dev, state, like, 2, monkeypatch)
+    probes_first = dev.probes
+    anchors = [a.data_ptr() for a in state.map.anchors]
+    assert first is not None and len(anchors) == 2 and state.searches == 1
+    second, pool2 = search(dev, state, like, 1, monkeypatch)
+    assert second is not None and state.searches == 2
+    assert [a.data_ptr() for a in state.map.anchors][:2] == anchors  # nothing was rediscovered
+    # the second search never measured a same-group reference pair again, and it found the
+    # groups' reference buffers in place: it only classified blocks and the model sample
+    assert pool2.map is pool1.map
+    for t, ref in zip(second[0], like):
+        assert dev.group_at(t) == dev.group_at(t, last=True) != dev.group_at(ref)
+    spans = sorted((t.data_ptr(), t.data_ptr() + t.numel() * 4) for col in (*first, *second) for t in col)
+    assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(spans, spans[1:])), "buffers overlap"
+    assert dev.probes - probes_first < probes_first
+
+
+def test_blocks_known_by_address_are_not_probed_again(small_constants, monkeypatch):
+    """Blocks a dropped wrapper returns to torch's cache come back at the same addresses: as long
+    as the allocator has given nothing back to the driver they are known without a probe."""
+
+    class Recycling(FakeDevice):
+        """Hands previously returned blocks out again first, like torch's caching allocator."""
+
+        def __init__(self, *a, **k):
+            super().__init__(*a, **k)
+            self.cache = []
+
+        def allocate(self, nbytes):
+            for i, t in enumerate(self.cache):
+                if t.numel() == nbytes:
+                    return self.cache.pop(i)
+            return super().allocate(nbytes)
+
+    dev = Recycling(total=160 * MiB, group_bytes=32 * MiB)
+    like = model_on(dev, [MiB // 2, MiB // 2])
+    state = H.DeviceState(torch.device("cpu"))
+    first, pool1 = search(dev, state, like, 2, monkeypatch)
+    probes_first = dev.probes
+    blocks = [b.storage for b in pool1.blocks if b.used > 0 and b not in state.anchor_blocks]
+    assert blocks
+    del first
+    dev.cache = list(blocks)  # the wrapper died: its blocks are cached, nothing went to the driver
+    second, pool2 = search(dev, state, like, 2, monkeypatch)
+    assert second is not None and pool2.cache_hits >= 1
+    # only the model sample was measured
+    assert dev.probes - probes_first <= 0.25 * probes_first
+    # ... but once memory has gone back to the driver the addresses are forgotten
+    dev.released += 1
+    pool3 = make_pool(dev, monkeypatch, state=state)
+    assert state.known == {} and pool3.cache_hits == 0
+
+
+def test_two_threads_search_one_at_a_time(small_constants, monkeypatch):
+    import threading
+
+    dev = FakeDevice(total=256 * MiB, group_bytes=48 * MiB)
+    busy = threading.Lock()
+    overlaps = []
+    plain = dev.probe_ms
+
+    def exclusive_probe(a, b, nbytes=None, repeats=3):
+        if not busy.acquire(blocking=False):
+            overlaps.append(1)
+            return plain(a, b, nbytes, repeats)
+        try:
+            return plain(a, b, nbytes, repeats)
+        finally:
+            busy.release()
+
+    dev.probe_ms = exclusive_probe
+    models = [model_on(dev, [MiB // 2, MiB // 2, 100]) for _ in range(2)]
+    state = H.DeviceState(torch.device("cpu"))
+    results = [None, None]
+
+    def construct(k):
+        results[k] = search(dev, state, models[k], 2, monkeypatch)[0]
+
+    threads = [threading.Thread(target=construct, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not overlaps, "two searches probed at the same time"
+    assert all(r is not None for r in results) and state.searches == 2
+    spans = sorted((t.data_ptr(), t.data_ptr() + t.numel() * 4) for r in results for col in r for t in col)
+    assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(spans, spans[1:])), "buffers overlap"
+    for r, like in zip(results, models):
+        for col in r:
+            for t, ref in zip(col, like):
+                assert dev.group_at(t) != dev.group_at(ref)
+
+
+def test_the_search_never_holds_more_than_its_allowance(small_constants, monkeypatch):
+    dev = FakeDevice(total=160 * MiB, group_bytes=32 * MiB)
+    like = model_on(dev, [MiB // 2, MiB // 2])   # 4 MiB at the start of group 0: 28 MiB to walk
+    held = []
+    plain = dev.allocate
+
+    def counting(nbytes):
+        t = plain(nbytes)
+        held.append(nbytes)
+        return t
+
+    dev.allocate = counting
+    state = H.DeviceState(torch.device("cpu"))
+    copies, pool = search(dev, state, like, 2, monkeypatch, limit=10 * MiB)
+    # ten blocks of 1 MiB do not reach the next group: no placement, and no more was taken
+    assert copies is None
+    assert sum(held) <= 10 * MiB
+    assert state.structured  # not a verdict on the device: a later search may get further
+    # with room to walk the same state carries on from its first anchor
+    copies, pool = search(dev, state, like, 2, monkeypatch, limit=64 * MiB)
+    assert copies is not None and len(state.map.anchors) == 2
+
+
+def test_the_allowance_follows_the_environment(monkeypatch):
+    assert H.search_limit_bytes(100 << 30) == 75 << 30
+    monkeypatch.setenv("TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB", "16")
+    assert H.search_limit_bytes(100 << 30) == 16 << 30
+    monkeypatch.setenv("TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB", "1000")
+    assert H.search_limit_bytes(100 << 30) == 75 << 30   # never more than the default share
+    monkeypatch.setenv("TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB", "lots")
+    assert H.search_limit_bytes(100 << 30) == 75 << 30
+
+
+def test_a_model_of_many_tensors_is_classified_from_a_sample(small_constants, monkeypatch):
+    dev = FakeDevice(total=400 * MiB, group_bytes=100 * MiB)
+    # 60 probe-able tensors of 2 MiB: 0-49 in group 0, 50-59 in group 1
+    like = model_on(dev, [MiB // 2] * 60)
+    truth = [dev.group_at(t) for t in like]
+    assert truth.count(0) == 50 and truth.count(1) == 10
+    pool = make_pool(dev, monkeypatch)
+    pool.grow_until(lambda pl: len(pl.map.anchors) >= 3)
+    before = dev.probes
+    groups = H.groups_of_tensors(pool, like)
+    measured = (dev.probes - before) / len(pool.map.anchors)
+    assert measured <= 5 + 8, "a sample and one bisection, not one probe per tensor"
+    names = {truth[0]: groups[0], truth[-1]: groups[-1]}
+    assert [names[g] for g in truth] == groups

@@ -6,7 +6,9 @@ concurrently slow each other down when they lie in the same group: a pair of
 in-place (read + write) streams runs at 5.6 TB/s inside one group against
 6.4 TB/s across two, two pure write streams at 5.8 against 7.1 TB/s, and a
 LocalSGD average whose parameters and backup share a group at 0.79 of the
-8 TB/s peak against 0.85 when they do not.  Read-only streams do not care.
+8 TB/s peak against 0.85 when they do not.  Read-only streams do not care (a
+plain copy runs at the same speed whether source and destination share a group
+or not).
 
 The replica-sync kernels write the live parameters, the backup and the outer
 momentum at the same element offsets at the same time.  Measured over the
@@ -25,8 +27,25 @@ buffers are allocated here, so this module
   while copying it into a scratch buffer, and runs 18-20 % longer when both lie
   in one group;
 * hands out per-tensor buffers from blocks of device memory whose group is
-  known (:class:`GroupedPool`): every tensor's backup and momentum in the group
-  after its parameter's.
+  known (:class:`GroupedPool`): every tensor's copies in a group other than its
+  parameter's, all copies of one tensor together.
+
+What is learnt about a device is kept for the life of the process
+(:class:`DeviceState`): one reference buffer ("anchor") per group found, and the
+group of every block the search has classified, valid for as long as torch's
+allocator has not returned memory to the driver.  A search runs under the
+device's lock, so two replicas that construct their wrappers at the same time
+on one GPU take turns instead of disturbing each other's timings.  A search
+takes device memory from torch in blocks of 2 GiB, holds what it cannot use
+until it is over (the driver hands physical memory out in address order: the
+way to the next group leads through the rest of the current one) and then
+gives it back; what it may hold at any time is bounded by
+``TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB`` (default: three quarters of the memory
+that is free when it starts).  While it runs, other allocations on the device
+see that much less free memory.  Which group the model's own tensors lie in is
+found by probing a handful of them (the probe rewrites them with their own
+contents; nothing else may write them meanwhile - the same moment at which the
+wrapper takes its first backup of them).
 
 Nothing here affects results: a wrong or impossible placement only costs
 bandwidth.  ``TORCHFT_AMD_HBM_PLACEMENT=0`` switches the probing off, and it is
@@ -36,9 +55,10 @@ group structure (other GPUs).
 
 from __future__ import annotations
 
-import ctypes
 import logging
 import os
+import threading
+import time
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
@@ -50,6 +70,7 @@ from .multi_tensor import current_stream_handle
 logger: logging.Logger = logging.getLogger(__name__)
 
 N_GROUPS = 3
+MAX_COPIES = 3               # backup, outer momentum, pseudo-gradients
 PROBE_BYTES = 512 << 20      # per buffer and probe: long enough to time reliably (0.3 ms), short enough to be free
 MIN_PROBE_BYTES = 128 << 20  # tensors below this are not probed (they take their neighbour's group)
 BLOCK_BYTES = 2 << 30        # device memory is taken from torch in blocks of this size
@@ -61,11 +82,28 @@ AMBIGUOUS_BAND = 0.03        # a ratio this close to the threshold is measured a
 RELATIVE_CONTRAST = 1.06     # own-group probe time / next longest, with all three anchors known
 NO_STRUCTURE_BYTES = 110 << 30  # this much memory in ONE group: the device has no such groups
 MIN_MODEL_BYTES = 256 << 20  # smaller models are left alone (a GPT-2-small of 0.5 GB still gains 1-2 %)
+MODEL_SAMPLES = 5            # tensors of the model probed before any bisection
+SEARCH_FRACTION = 0.75       # of the free device memory a search may hold, unless the environment says
 ALIGN = 256
+
+#: probe launches issued by this process (all devices); tests and logs read it
+launch_count = 0
 
 
 def enabled() -> bool:
     return os.environ.get("TORCHFT_AMD_HBM_PLACEMENT", "1") not in ("0", "false", "off")
+
+
+def search_limit_bytes(free_bytes: int) -> int:
+    """Most device memory one search may hold at a time."""
+    limit = int(free_bytes * SEARCH_FRACTION)
+    env = os.environ.get("TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB")
+    if env:
+        try:
+            limit = min(limit, int(float(env) * (1 << 30)))
+        except ValueError:
+            logger.warning("TORCHFT_AMD_HBM_PLACEMENT_MAX_GIB=%r is not a number; ignored", env)
+    return limit
 
 
 def _as_bytes(t: torch.Tensor) -> torch.Tensor:
@@ -75,7 +113,8 @@ def _as_bytes(t: torch.Tensor) -> torch.Tensor:
 def probe_ms(a: torch.Tensor, b: torch.Tensor, nbytes: Optional[int] = None, repeats: int = 3) -> float:
     """Shortest of ``repeats`` timings of the pair probe over the first ``nbytes`` bytes of
     ``a`` and ``b`` (default: as much as both hold, at most PROBE_BYTES).  ``a`` keeps its
-    contents (nothing else may touch it meanwhile); ``b`` is scratch and is overwritten."""
+    contents (nothing else may write it meanwhile); ``b`` is scratch and is overwritten."""
+    global launch_count
     a8, b8 = _as_bytes(a), _as_bytes(b)
     n = min(a8.numel(), b8.numel(), PROBE_BYTES if nbytes is None else nbytes)
     # 16-byte alignment of both ends
@@ -96,17 +135,19 @@ def probe_ms(a: torch.Tensor, b: torch.Tensor, nbytes: Optional[int] = None, rep
             stop.record()
             stop.synchronize()
             best = min(best, start.elapsed_time(stop))
+            launch_count += 1
     return best
 
 
-@dataclass
+@dataclass(eq=False)  # compared by identity: a block is a piece of device memory
 class _Block:
     storage: torch.Tensor  # uint8, BLOCK_BYTES (or larger for a tensor that needs it)
     group: int
     used: int = 0
+    floor: int = 0         # bytes at the start that are never handed out (an anchor lives there)
 
     def free(self) -> int:
-        return self.storage.numel() - self.used
+        return self.storage.numel() - max(self.used, self.floor)
 
 
 @dataclass
@@ -137,26 +178,75 @@ class GroupMap:
         the anchor of ``t``'s own group takes clearly longer than against the other two,
         whatever constant a profiler or a busy host adds to every launch.  Before that, the
         probe times are compared with the time of a pair that certainly shares a group.
-        An unclear measurement is repeated with more launches."""
+        A first pass with one timed launch per anchor settles the clear cases; an unclear
+        measurement is repeated with more launches."""
         size = _as_bytes(t).numel()
         n = min(size, PROBE_BYTES if nbytes is None else nbytes) // 16 * 16
         if n < MIN_PROBE_BYTES or not self.anchors:
             return None
-        for repeats in (3, 6, 9):
+        relative = len(self.anchors) >= N_GROUPS
+        best, ratio = 0, 0.0
+        for repeats in ((1, 3, 6, 9) if relative else (3, 6, 9)):
             times = [probe_ms(t, anchor, n, repeats) for anchor in self.anchors]
             best = max(range(len(times)), key=lambda k: times[k])
-            if len(self.anchors) >= N_GROUPS:
+            if relative:
                 second = max(x for k, x in enumerate(times) if k != best)
-                contrast = times[best] / second
-                if contrast > RELATIVE_CONTRAST:
+                # a single timed launch has to be clearer than the repeated measurement
+                margin = RELATIVE_CONTRAST + (0.04 if repeats == 1 else 0.0)
+                if times[best] / second > margin:
                     return best
                 continue  # no anchor stands out: measure again
             ratio = times[best] / self._same_ms(n)
             if abs(ratio - SAME_GROUP_RATIO) > AMBIGUOUS_BAND:
                 return best if ratio > SAME_GROUP_RATIO else None
-        if len(self.anchors) >= N_GROUPS:
+        if relative:
             return None
         return best if ratio > SAME_GROUP_RATIO else None
+
+
+class DeviceState:
+    """What this process knows about one device's bank groups, kept until it exits."""
+
+    def __init__(self, device: torch.device) -> None:
+        self.device = device
+        self.lock = threading.RLock()
+        self.map = GroupMap(device)
+        # blocks whose first PROBE_BYTES are an anchor: never returned; the rest of each is
+        # handed out once (it is not reclaimed when the tensors carved from it die)
+        self.anchor_blocks: List[_Block] = []
+        # address of a block classified earlier -> (bytes, group); valid while torch's
+        # allocator has not given memory back to the driver since (``epoch``)
+        self.known: Dict[int, Tuple[int, int]] = {}
+        self.epoch: Optional[int] = None
+        self.structured = True   # False once the timings have shown no group structure
+        self.searches = 0
+
+
+_STATES: Dict[Tuple[str, int], DeviceState] = {}
+_STATES_LOCK = threading.Lock()
+
+
+def device_state(device: torch.device) -> DeviceState:
+    index = device.index if device.index is not None else (
+        torch.cuda.current_device() if device.type == "cuda" else 0)
+    key = (device.type, index)
+    with _STATES_LOCK:
+        state = _STATES.get(key)
+        if state is None:
+            state = _STATES[key] = DeviceState(torch.device(device.type, index))
+        return state
+
+
+def forget_devices() -> None:
+    """Drops everything learnt (anchors included).  For tests."""
+    with _STATES_LOCK:
+        _STATES.clear()
+
+
+def _device_free_count(device: torch.device) -> int:
+    """How often torch's allocator has returned a segment to the driver: as long as this does
+    not change, an address that was classified still names the same physical memory."""
+    return int(torch.cuda.memory_stats(device).get("num_device_free", 0))
 
 
 class GroupedPool:
@@ -164,7 +254,8 @@ class GroupedPool:
 
     Blocks come from torch's allocator (so they are accounted for and returned like any
     other tensor): ``grow_until`` takes them, ``take`` carves tensors out of them,
-    ``release_unused`` returns the untouched ones.
+    ``release_unused`` returns the untouched ones.  A pool serves one search; what outlives
+    it (anchors, classified addresses) lives in the :class:`DeviceState` it was given.
     """
 
     def __init__(
@@ -173,26 +264,42 @@ class GroupedPool:
         allocate: Optional[Callable[[int], torch.Tensor]] = None,
         free_memory: Optional[Callable[[], int]] = None,
         release: Optional[Callable[[], None]] = None,
+        state: Optional[DeviceState] = None,
+        epoch: Optional[Callable[[], int]] = None,
     ) -> None:
         self.device = device
-        self.map = GroupMap(device)
-        self.blocks: List[_Block] = []
+        self.state = state if state is not None else DeviceState(device)
+        self.map = self.state.map
+        # the unreserved rest of the anchors' blocks is the first memory of known group
+        self.blocks: List[_Block] = list(self.state.anchor_blocks)
         self._straddling: List[torch.Tensor] = []  # blocks across a group boundary: held, unused
-        self.structured = True  # False once the timings show no group structure
         # where blocks come from and go back to (replaceable: the search logic is host code
         # and is tested without a GPU)
         self._allocate = allocate or (lambda n: torch.empty(n, dtype=torch.uint8, device=device))
         self._free_memory = free_memory or (lambda: torch.cuda.mem_get_info(device)[0])
         self._release = release or torch.cuda.empty_cache
+        self._epoch = epoch or (
+            (lambda: _device_free_count(device)) if device.type == "cuda" else (lambda: 0))
         self.keep_free = 6 << 30  # device memory the search never touches
+        self.limit: Optional[int] = None  # bytes this search may hold; None: search_limit_bytes
+        self.held = 0             # bytes taken from the device by this search
+        self.cache_hits = 0
+        if self.state.epoch is not None and self.state.epoch != self._epoch():
+            self.state.known.clear()  # memory went back to the driver: addresses mean nothing now
+
+    @property
+    def structured(self) -> bool:
+        return self.state.structured
 
     # -- discovery ---------------------------------------------------------------
-    def _classify_block(self, storage: torch.Tensor) -> Optional[int]:
+    def _classify_block(self, block: _Block) -> Optional[int]:
         """Group of a fresh block (a new anchor is made of it if its group is new); None if
         the block straddles two groups."""
         m = self.map
+        storage = block.storage
         if not m.anchors:
             m.anchors.append(storage[:PROBE_BYTES])
+            self._keep_as_anchor(block)
             return 0
         n = storage.numel()
         ends = []
@@ -202,9 +309,19 @@ class GroupedPool:
                 if len(m.anchors) >= N_GROUPS or not self._clearly_new(storage):
                     return None  # matches no group clearly: leave it alone
                 m.anchors.append(piece)
+                self._keep_as_anchor(block, at_end=piece.data_ptr() != storage.data_ptr())
                 g = len(m.anchors) - 1
             ends.append(g)
         return ends[0] if ends[0] == ends[1] else None
+
+    def _keep_as_anchor(self, block: _Block, at_end: bool = False) -> None:
+        if at_end:
+            # the anchor is the block's tail (a block across a boundary founded the group):
+            # nothing of it is handed out
+            block.floor = block.storage.numel()
+        else:
+            block.floor = min(PROBE_BYTES, block.storage.numel())
+        self.state.anchor_blocks.append(block)
 
     def _clearly_new(self, storage: torch.Tensor) -> bool:
         """A second, longer measurement before a block founds a new group: an anchor that in
@@ -220,26 +337,44 @@ class GroupedPool:
 
     def grow_until(self, satisfied, keep_free: Optional[int] = None, block_bytes: Optional[int] = None) -> bool:
         """Takes blocks from the device, one at a time, until ``satisfied(self)`` holds; False if
-        the device ran out first.  Every block that lies in one group is kept as a candidate
-        (the driver hands physical memory out in address order, so the way to the next group
-        leads through the rest of the current one: what is not wanted must be held, not
-        returned, until the search is over - ``release_unused`` gives it back)."""
+        the device, or the search's allowance, ran out first.  Every block that lies in one
+        group is kept as a candidate (the driver hands physical memory out in address order,
+        so the way to the next group leads through the rest of the current one: what is not
+        wanted must be held, not returned, until the search is over - ``release_unused``
+        gives it back)."""
         keep_free = self.keep_free if keep_free is None else keep_free
         block_bytes = BLOCK_BYTES if block_bytes is None else block_bytes
+        if self.limit is None:
+            self.limit = search_limit_bytes(max(self._free_memory() - keep_free, 0))
         while not satisfied(self):
+            if not self.state.structured:
+                return False
             if self._free_memory() < keep_free + block_bytes:
                 logger.info("hbm placement: device memory ran out before the search was satisfied")
                 return False
+            if self.held + block_bytes > self.limit:
+                logger.info("hbm placement: the search stops at its allowance of %.1f GiB",
+                            self.limit / (1 << 30))
+                return False
             storage = self._allocate(block_bytes)
-            g = self._classify_block(storage)
+            self.held += block_bytes
+            block = _Block(storage, -1)
+            cached = self.state.known.get(storage.data_ptr())
+            if cached is not None and cached[0] == storage.numel() and cached[1] < len(self.map.anchors):
+                g: Optional[int] = cached[1]
+                self.cache_hits += 1
+            else:
+                g = self._classify_block(block)
             if g is None:
                 self._straddling.append(storage)
             else:
-                self.blocks.append(_Block(storage, g))
-            if len(self.map.anchors) == 1 and len(self.blocks) * block_bytes > NO_STRUCTURE_BYTES:
+                block.group = g
+                self.blocks.append(block)
+                self.state.known[storage.data_ptr()] = (storage.numel(), g)
+            if len(self.map.anchors) == 1 and self.held > NO_STRUCTURE_BYTES:
                 # more than a whole group's worth of memory and still one group: this
                 # device shows no group structure
-                self.structured = False
+                self.state.structured = False
                 return False
         return True
 
@@ -251,7 +386,7 @@ class GroupedPool:
             for b in self.blocks:
                 if b.group != g:
                     continue
-                start = -(-b.used // ALIGN) * ALIGN
+                start = -(-max(b.used, b.floor) // ALIGN) * ALIGN
                 if start + nbytes <= b.storage.numel():
                     b.used = start + nbytes
                     return b.storage[start:start + nbytes]
@@ -263,41 +398,81 @@ class GroupedPool:
             b.used = 0
 
     def release_unused(self) -> None:
-        """Gives every block nothing was taken from back to the device."""
-        self.blocks = [b for b in self.blocks if b.used > 0]
+        """Gives every block nothing was taken from back to the device (anchors stay)."""
+        anchors = self.state.anchor_blocks
+        for b in self.blocks:
+            if b.used == 0 and b not in anchors:
+                self.state.known.pop(b.storage.data_ptr(), None)
+        self.blocks = [b for b in self.blocks if b.used > 0 or b in anchors]
         self._straddling = []
+        self.held = 0
         self._release()
+        self.state.epoch = self._epoch()
+
+
+def _sample_groups(pool: GroupedPool, tensors: Sequence[torch.Tensor], probeable: List[int],
+                   out: List[Optional[int]]) -> None:
+    """Fills ``out`` for the probe-able tensors.  A model's tensors are allocated one after
+    the other, so they lie in at most a few runs of one group each: a handful of probes
+    spread over the list, then bisection between neighbours that disagree, instead of one
+    probe per tensor."""
+    def probe(k: int) -> Optional[int]:
+        i = probeable[k]
+        if out[i] is None:
+            out[i] = pool.map.group_of(tensors[i])
+            probed.add(k)
+        return out[i]
+
+    probed: set = set()
+    n = len(probeable)
+    if n == 0:
+        return
+    picks = sorted({round(j * (n - 1) / max(MODEL_SAMPLES - 1, 1)) for j in range(MODEL_SAMPLES)})
+    for k in picks:
+        probe(k)
+    # bisect between sampled neighbours whose groups differ
+    work = list(zip(picks, picks[1:]))
+    while work:
+        lo, hi = work.pop()
+        if hi - lo <= 1 or out[probeable[lo]] == out[probeable[hi]]:
+            continue
+        mid = (lo + hi) // 2
+        probe(mid)
+        work += [(lo, mid), (mid, hi)]
+    # everything in between takes the group of the nearest probed tensor in list order
+    known = sorted(probed)
+    for k in range(n):
+        if k not in probed:
+            nearest = min(known, key=lambda j: (abs(j - k), j))
+            out[probeable[k]] = out[probeable[nearest]]
 
 
 def groups_of_tensors(pool: GroupedPool, tensors: Sequence[torch.Tensor]) -> List[Optional[int]]:
-    """Bank group of every tensor (against the pool's anchors); tensors too small to probe
-    take the group of the nearest probed tensor by address."""
+    """Bank group of every tensor (against the pool's anchors).  Of the tensors large enough
+    to probe a sample is measured (see ``_sample_groups``); tensors too small to probe take
+    the group of the nearest classified tensor by address."""
     out: List[Optional[int]] = [None] * len(tensors)
-    probed: List[Tuple[int, int]] = []  # (address, group)
-    for i, t in enumerate(tensors):
-        if _as_bytes(t).numel() >= MIN_PROBE_BYTES:
-            g = pool.map.group_of(t)
-            out[i] = g
-            if g is not None:
-                probed.append((t.data_ptr(), g))
-    if probed:
+    probeable = [i for i, t in enumerate(tensors) if _as_bytes(t).numel() >= MIN_PROBE_BYTES]
+    _sample_groups(pool, tensors, probeable, out)
+    placed = [(tensors[i].data_ptr(), out[i]) for i in probeable if out[i] is not None]
+    if placed:
         for i, t in enumerate(tensors):
             if out[i] is None and _as_bytes(t).numel() < MIN_PROBE_BYTES:
                 addr = t.data_ptr()
-                out[i] = min(probed, key=lambda ag: abs(ag[0] - addr))[1]
+                out[i] = min(placed, key=lambda ag: abs(ag[0] - addr))[1]
     return out
 
 
 def allocate_apart(
     like: Sequence[torch.Tensor], n_copies: int
 ) -> Optional[List[List[torch.Tensor]]]:
-    """``n_copies`` (1 or 2) sets of uninitialised tensors shaped like ``like``, every tensor
-    of every copy in the bank group after its model tensor's: group (g + 1) mod 3, where g
-    is the group of the corresponding tensor of ``like``; what does not fit there goes to
-    group (g + 2) mod 3, and only then to g itself.  Returns None when placement does not
-    apply (switched off, not on a GPU, model too small, no group structure found); the
-    caller then allocates as it always did."""
-    if not enabled() or not like or n_copies not in (1, 2):
+    """``n_copies`` (1 to 3) sets of uninitialised tensors shaped like ``like``, every tensor
+    of every copy in a bank group other than its model tensor's: the group after it in
+    order of discovery; what does not fit there goes to the remaining group, and only then
+    to the tensor's own.  Returns None when placement does not apply (switched off, not on
+    a GPU, model too small, no group structure found); the caller then allocates as it
+    always did."""
+    if not enabled() or not like or not 1 <= n_copies <= MAX_COPIES:
         return None
     device = like[0].device
     if device.type != "cuda" or any(t.device != device for t in like):
@@ -305,50 +480,73 @@ def allocate_apart(
     sizes = [t.numel() * t.element_size() for t in like]
     if sum(sizes) < MIN_MODEL_BYTES:
         return None
-    try:
-        return _allocate_apart(like, sizes, n_copies, device)
-    except Exception as e:  # placement is an optimisation: never let it fail an allocation
-        logger.warning("hbm placement gave up (%s); default allocation", e)
-        torch.cuda.empty_cache()
-        return None
+    return _locked_search(device_state(device), like, sizes, n_copies, device)
+
+
+def _locked_search(
+    state: DeviceState, like: Sequence[torch.Tensor], sizes: List[int], n_copies: int,
+    device: torch.device, make_pool: Optional[Callable[[DeviceState], "GroupedPool"]] = None,
+) -> Optional[List[List[torch.Tensor]]]:
+    """One search at a time per device: concurrent probes would disturb each other's timings,
+    and two searches would each hold the memory the other is looking for."""
+    with state.lock:
+        if not state.structured:
+            return None
+        try:
+            pool = make_pool(state) if make_pool is not None else None
+            return _allocate_apart(like, sizes, n_copies, device, pool=pool, state=state)
+        except Exception as e:  # placement is an optimisation: never let it fail an allocation
+            logger.warning("hbm placement gave up (%s); default allocation", e)
+            if device.type == "cuda":
+                torch.cuda.empty_cache()
+            return None
 
 
 def _allocate_apart(
     like: Sequence[torch.Tensor], sizes: List[int], n_copies: int, device: torch.device,
-    pool: Optional[GroupedPool] = None,
+    pool: Optional[GroupedPool] = None, state: Optional[DeviceState] = None,
 ) -> Optional[List[List[torch.Tensor]]]:
+    global launch_count
+    t0, launches0 = time.perf_counter(), launch_count
     if pool is None:
         torch.cuda.synchronize(device)
-        pool = GroupedPool(device)
+        pool = GroupedPool(device, state=state)
+    pool.state.searches += 1
     largest = max(sizes)
     block = max(BLOCK_BYTES, -(-largest // BLOCK_GRANULE) * BLOCK_GRANULE)
-    # first: reach all groups, so that there is an anchor to compare the model with in each
-    pool.grow_until(lambda pl: len(pl.map.anchors) >= N_GROUPS, block_bytes=block)
+    # first: two groups, so that there is somewhere else to go and something to compare with
+    pool.grow_until(lambda pl: len(pl.map.anchors) >= 2, block_bytes=block)
     if not pool.structured or len(pool.map.anchors) < 2:
         logger.info("hbm placement: no bank-group structure found on %s; default allocation", device)
+        if not pool.structured:
+            # nothing to compare with on this device, now or later: keep nothing
+            pool.map.anchors.clear()
+            pool.state.anchor_blocks.clear()
+            pool.blocks = []
         pool.release_unused()
         return None
-    n_groups = len(pool.map.anchors)
+    n_known = len(pool.map.anchors)
     groups = groups_of_tensors(pool, like)
-    need: Dict[int, int] = {g: 0 for g in range(n_groups)}
-    wanted: List[List[int]] = []
-    for size, g in zip(sizes, groups):
-        g0 = 0 if g is None else g
-        row = [(g0 + 1) % n_groups] * n_copies
-        wanted.append(row)
-        for w in row:
-            need[w] += -(-size // ALIGN) * ALIGN
+    # a tensor in none of the known groups lies in the one not reached yet: every known group
+    # is "another group" for it; the first is as good as any
+    wanted = [((0 if g is None else g + 1) % n_known) for g in groups]
+    need: Dict[int, int] = {}
+    for size, w in zip(sizes, wanted):
+        need[w] = need.get(w, 0) + n_copies * (-(-size // ALIGN) * ALIGN)
     # head room for blocks that cannot be filled to the last byte
     need = {g: n + block for g, n in need.items() if n > 0}
     pool.grow_until(lambda pl: all(pl.free_bytes(g) >= n for g, n in need.items()), block_bytes=block)
-    copies: List[List[torch.Tensor]] = [[] for _ in range(n_copies)]
+    n_groups = len(pool.map.anchors)
     order = sorted(range(len(like)), key=lambda i: -sizes[i])  # large tensors first: they pack better
     placed: Dict[Tuple[int, int], Optional[torch.Tensor]] = {}
     misplaced = 0
     for i in order:
+        prefer = wanted[i]
+        own = groups[i]
+        others = [g for g in range(n_groups) if g != prefer and g != own]
+        if own is not None and own != prefer:
+            others.append(own)  # the tensor's own group last
         for k in range(n_copies):
-            prefer = wanted[i][k]
-            others = [(prefer + 1) % n_groups, (prefer + 2) % n_groups][: n_groups - 1]
             raw = pool.take(sizes[i], [prefer]) if sizes[i] else None
             if raw is None and sizes[i]:
                 raw = pool.take(sizes[i], others)
@@ -356,16 +554,18 @@ def _allocate_apart(
             placed[(i, k)] = raw
     # everything the search held but did not use goes back BEFORE anything else is allocated:
     # what found no room in the pool must not fail for memory the pool itself is sitting on
+    held = pool.held
     pool.release_unused()
     for (i, k), raw in list(placed.items()):
         if raw is None:
             raw = pool._allocate(max(sizes[i], 1))[: sizes[i]]
         placed[(i, k)] = raw.view(like[i].dtype).view(like[i].shape)
-    for k in range(n_copies):
-        copies[k] = [placed[(i, k)] for i in range(len(like))]
+    copies = [[placed[(i, k)] for i in range(len(like))] for k in range(n_copies)]
     logger.info(
-        "hbm placement: %d tensors x %d copies over %d bank groups (%d not in their preferred group)",
-        len(like), n_copies, n_groups, misplaced,
+        "hbm placement: %d tensors x %d copies over %d bank groups (%d not in their preferred group); "
+        "search %d on %s: %.2f s, %d probe launches, %d blocks known by address, %.1f GiB held at most",
+        len(like), n_copies, n_groups, misplaced, pool.state.searches, device,
+        time.perf_counter() - t0, launch_count - launches0, pool.cache_hits, held / (1 << 30),
     )
     return copies
 
@@ -373,7 +573,7 @@ def _allocate_apart(
 def model_copies(like: Sequence[torch.Tensor], n_copies: int) -> List[List[torch.Tensor]]:
     """``n_copies`` sets of uninitialised tensors shaped like ``like``: placed by bank group
     where that applies (:func:`allocate_apart`), otherwise one plain allocation per tensor."""
-    placed = allocate_apart(like, n_copies) if n_copies in (1, 2) else None
+    placed = allocate_apart(like, n_copies) if 1 <= n_copies <= MAX_COPIES else None
     if placed is not None:
         return placed
     return [[torch.empty_like(t) for t in like] for _ in range(n_copies)]

@@ -29,6 +29,8 @@ With a Manager that is not this package's (for instance a mock) the per-paramete
 from __future__ import annotations
 
 import logging
+import operator
+from dataclasses import dataclass
 from types import TracebackType
 from typing import Dict, List, Optional, Sequence, Tuple, Type
 
@@ -44,6 +46,39 @@ logger: logging.Logger = logging.getLogger(__name__)
 
 
 _KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+_DATA_PTR = torch.Tensor.data_ptr
+_NUMEL = torch.Tensor.numel
+_MOMENTUM_OF = operator.itemgetter("momentum_buffer")
+
+
+@dataclass
+class _Bound:
+    """The tensors a wrapper synchronises, gathered once and re-validated on every sync by
+    address and size alone (C-level maps over the parameter objects), so that a sync does
+    not walk the module tree or create 2 x T tensor objects again.  ``generation`` changes
+    whenever the lists are rebuilt; everything derived from them is keyed on it."""
+
+    generation: int
+    names: List[str]
+    params: List[torch.Tensor]       # p.data of every parameter
+    backups: List[torch.Tensor]
+    backup_dict: Dict[str, torch.Tensor]
+    param_key: Tuple
+    backup_key: Tuple
+    on_device: bool = False          # parameters and backups all on one GPU
+
+
+@dataclass
+class _SgdPlan:
+    """What ``_fusable_sgd`` found, and what it has to be compared with to still hold."""
+
+    entries: Optional[List[Tuple[List[int], "ops.OuterSGD", bool]]]
+    state: object                    # the optimizer's state mapping itself
+    n_state: int
+    groups_key: Tuple
+    bufs: Optional[List[Optional[torch.Tensor]]]   # momentum buffers found, by parameter index
+    slots: Optional[List[dict]]      # optimizer.state[p] of every parameter (steady state)
 
 
 def _is_native_manager(manager: object) -> bool:
@@ -141,9 +176,16 @@ class LocalSGD:
         self._host_backup: Optional[_PackedHostBackup] = None
         self._hooks: List[RemovableHandle] = []
         self._tables: Dict[str, TensorTable] = {}
+        self._launches: Dict[str, tuple] = {}  # prepared launches, with what they were prepared for
         self._flat: Dict[str, tuple] = {}
-        self._placed_momentum: Optional[List[torch.Tensor]] = None
+        self._placed_momentum: Optional[List[Optional[torch.Tensor]]] = None
+        self._placed_grads: Optional[List[torch.Tensor]] = None
         named = list(self._model.named_parameters())
+        # like an optimizer, the wrapper binds to the parameters the model has now
+        self._param_names: List[str] = [name for name, _ in named]
+        self._param_objs: List[nn.Parameter] = [p for _, p in named]
+        self._bound: Optional[_Bound] = None
+        self._generation = 0
         if (
             backup_device is not None
             and torch.device(backup_device).type == "cpu"
@@ -168,7 +210,7 @@ class LocalSGD:
             placed = hbm_placement.allocate_apart(datas, self._placed_copies())
             if placed is not None:
                 views = placed[0]
-                self._placed_momentum = placed[1] if len(placed) > 1 else None
+                self._keep_placed(placed[1:])
             else:
                 _, views = self._flat_like("backup", datas)
             for (name, _), view in zip(named, views):
@@ -196,6 +238,9 @@ class LocalSGD:
     def _placed_copies(self) -> int:
         """Model-sized device buffers this wrapper will keep: the backup."""
         return 1
+
+    def _keep_placed(self, extra: Sequence[List[torch.Tensor]]) -> None:
+        """Receives the copies allocated together with the backup (none for LocalSGD)."""
 
     # -- context manager / hook ---------------------------------------------
     def __enter__(self) -> "LocalSGD":
@@ -225,12 +270,32 @@ class LocalSGD:
 
     # -- tensors -------------------------------------------------------------
     def _named(self) -> Tuple[List[str], List[torch.Tensor], List[torch.Tensor]]:
-        names, params, backups = [], [], []
-        for name, p in self._model.named_parameters():
-            assert name in self._backup_parameters
-            names.append(name)
-            params.append(p.data)
-            backups.append(self._backup_parameters[name])
+        """(names, parameter data, backups) in ``named_parameters()`` order.  The lists are
+        kept between syncs and only rebuilt when a parameter or a backup tensor has moved
+        (``p.data`` reassigned, ``_backup_parameters`` replaced or refilled by the user)."""
+        objs = self._param_objs
+        backup_dict = self._backup_parameters
+        param_key = (tuple(map(_DATA_PTR, objs)), tuple(map(_NUMEL, objs)))
+        backup_key = tuple(map(_DATA_PTR, backup_dict.values()))
+        bound = self._bound
+        if (
+            bound is not None
+            and bound.param_key == param_key
+            and bound.backup_dict is backup_dict
+            and bound.backup_key == backup_key
+        ):
+            return bound.names, bound.params, bound.backups
+        names = self._param_names
+        backups = []
+        for name in names:
+            assert name in backup_dict
+            backups.append(backup_dict[name])
+        self._generation += 1
+        params = [p.data for p in objs]
+        self._bound = _Bound(
+            self._generation, names, params, backups, backup_dict, param_key, backup_key,
+            self._on_device(params, backups),
+        )
         return names, params, backups
 
     @staticmethod
@@ -296,10 +361,15 @@ class LocalSGD:
         self._local_step = 0
 
     def _fused(self, params: Sequence[torch.Tensor], backups: Sequence[torch.Tensor]) -> bool:
+        bound = self._bound
+        on_device = (
+            bound.on_device if bound is not None and bound.params is params
+            else self._on_device(params, backups)
+        )
         return (
-            _is_native_manager(self._manager)
+            on_device
+            and _is_native_manager(self._manager)
             and self._manager.supports_fused_sync()
-            and self._on_device(params, backups)
         )
 
     def _perform_sync(self) -> None:
@@ -326,28 +396,39 @@ class LocalSGD:
         reason other than the launch itself (the quorum, finding the peers' buffers,
         building and validating the tensor table) happens before the vote and is latched
         like a failed all-reduce; a launch that fails after the vote raises, because the
-        group has already counted the step as committed."""
+        group has already counted the step as committed.
+
+        The prepared launches are kept: as long as the parameters, the backups and the
+        peers' buffers are the ones of the previous sync, nothing is rebuilt or compared
+        tensor by tensor."""
         manager = self._manager
         manager.wait_quorum()  # should_commit reads the quorum's results (async quorum)
         launches = []
+        mask = 0
         if manager.errored() is None:
             try:
-                replicas, mask = manager.replica_columns(params)
-                for idx in ops.dtype_groups(params):
-                    outs = [[params[i] for i in idx], [backups[i] for i in idx]]
-                    reps = [[rep[i] for i in idx] for rep in replicas]
-                    key = f"average/{params[idx[0]].dtype}"
-                    table = self._tables.get(key)
-                    if table is None or not table.matches([*outs, *reps]):
-                        table = ops.reduce_avg_table(outs, reps)
-                    launches.append((key, outs, reps, mask, table))
+                generation = self._generation
+                replicas, mask = manager.replica_columns(params, identity=(id(self), generation))
+                kept = self._launches.get("average")
+                if kept is not None and kept[0] == generation and kept[1] is replicas:
+                    launches = kept[2]
+                else:
+                    for idx in ops.dtype_groups(params):
+                        outs = [[params[i] for i in idx], [backups[i] for i in idx]]
+                        reps = [[rep[i] for i in idx] for rep in replicas]
+                        key = f"average/{params[idx[0]].dtype}"
+                        table = self._tables.get(key)
+                        if table is None or not table.matches([*outs, *reps]):
+                            table = ops.reduce_avg_table(outs, reps)
+                        launches.append((key, outs, reps, table))
+                    self._launches["average"] = (generation, replicas, launches)
             except Exception as e:  # same latch as Manager.allreduce
                 logger.exception("got exception preparing the fused sync -- skipping: %s", e)
                 manager.report_error(e)
                 launches = []
         if manager.should_commit():
             assert launches, "a replica that failed to prepare cannot have voted to commit"
-            for key, outs, reps, mask, table in launches:
+            for key, outs, reps, table in launches:
                 self._tables[key] = ops.mt_reduce_avg(
                     outs, reps, mask, manager.num_participants(), table=table, table_is_current=True
                 )
@@ -366,7 +447,7 @@ class LocalSGD:
 
     def _average(self) -> None:
         works = []
-        for p in self._model.parameters():
+        for p in self._param_objs:
             works.append(self._manager.allreduce(p.data.detach()))
         for work in works:
             work.wait()
@@ -418,6 +499,19 @@ def _fusable_sgd(
     return plan
 
 
+_GROUP_FIELDS = ("momentum", "dampening", "weight_decay", "nesterov", "maximize", "differentiable")
+
+
+def _groups_key(optimizer: optim.Optimizer) -> Tuple:
+    """What ``_fusable_sgd`` reads from the parameter groups (an lr schedule changes it)."""
+    return tuple(
+        (id(g["params"]), len(g["params"]),
+         g["lr"] if not isinstance(g["lr"], torch.Tensor) else id(g["lr"]),
+         *[g.get(name) for name in _GROUP_FIELDS])
+        for g in optimizer.param_groups
+    )
+
+
 class DiLoCo(LocalSGD):
     """DiLoCo (https://arxiv.org/pdf/2311.08105): the replicas average their
     pseudo-gradients ``params - backup`` and an outer optimizer applies the average
@@ -439,15 +533,38 @@ class DiLoCo(LocalSGD):
                 "Ensure that the manager is initialized with use_async_quorum=False"
             )
         self._outer_optimizer = outer_optimizer  # before super().__init__: see _placed_copies
-        super().__init__(manager, model, inner_optimizer, sync_every, backup_device, pin_memory)
         self._grads: Optional[List[torch.Tensor]] = None
+        self._plan: Optional[_SgdPlan] = None
+        super().__init__(manager, model, inner_optimizer, sync_every, backup_device, pin_memory)
+
+    # -- buffers allocated with the backup ---------------------------------------
+    def _wants_momentum(self) -> bool:
+        opt = self._outer_optimizer
+        return type(opt) is optim.SGD and any(g.get("momentum", 0) != 0 for g in opt.param_groups)
+
+    def _wants_grad_buffers(self) -> bool:
+        """Whether a sync will materialise the averaged pseudo-gradients per parameter: not
+        when the whole step is one launch (they stay in registers), and not when the model
+        is bucketised into one flat buffer per dtype."""
+        manager = self._manager
+        if not _is_native_manager(manager):
+            return True  # the per-parameter manager.allreduce contract
+        if not manager.supports_fused_sync():
+            return False  # bucketised
+        return not (manager.reduction_fails_only_at_launch() and type(self._outer_optimizer) is optim.SGD)
 
     def _placed_copies(self) -> int:
-        """The backup, plus the outer momentum when a fusable SGD with momentum will create it."""
-        opt = self._outer_optimizer
-        if type(opt) is optim.SGD and any(g.get("momentum", 0) != 0 for g in opt.param_groups):
-            return 2
-        return 1
+        """The backup, plus the outer momentum when a fusable SGD with momentum will create it,
+        plus the pseudo-gradients where a sync needs them in memory: all found in ONE search
+        at construction, none inside a sync."""
+        return 1 + int(self._wants_momentum()) + int(self._wants_grad_buffers())
+
+    def _keep_placed(self, extra: Sequence[List[torch.Tensor]]) -> None:
+        extra = list(extra)
+        if self._wants_momentum() and extra:
+            self._placed_momentum = list(extra.pop(0))
+        if self._wants_grad_buffers() and extra:
+            self._placed_grads = extra.pop(0)
 
     def _grad_buffers(self, params: Sequence[torch.Tensor]) -> List[torch.Tensor]:
         """Pseudo-gradient storage, kept across syncs (the reference allocates it anew
@@ -456,39 +573,91 @@ class DiLoCo(LocalSGD):
             g.shape != p.shape or g.device != p.device or g.dtype != p.dtype
             for g, p in zip(self._grads, params)
         ):
-            # written next to the parameters by the pseudo-gradient launch: keep them out of
-            # the parameters' HBM bank group, like the backup
-            self._grads = hbm_placement.model_copies(params, 1)[0]
+            placed, self._placed_grads = self._placed_grads, None
+            if placed is not None and len(placed) == len(params) and all(
+                g.shape == p.shape and g.device == p.device and g.dtype == p.dtype
+                for g, p in zip(placed, params)
+            ):
+                # allocated with the backup, outside the parameters' HBM bank group (they are
+                # written next to the parameters by the pseudo-gradient launch)
+                self._grads = placed
+            else:
+                self._grads = [torch.empty_like(p) for p in params]
         return self._grads
+
+    # -- the outer optimizer -------------------------------------------------------
+    def _sgd_plan(self, params: Sequence[torch.Tensor]) -> Optional[List[Tuple[List[int], ops.OuterSGD, bool]]]:
+        """``_fusable_sgd`` of the outer optimizer, recomputed only when something it depends
+        on has changed: the parameters (generation), the groups' hyper-parameters, the
+        optimizer's state mapping (replaced by ``load_state_dict``, grown or cleared), or a
+        momentum buffer in it."""
+        opt = self._outer_optimizer
+        plan = self._plan
+        groups_key = (self._generation, _groups_key(opt))
+        if (
+            plan is not None
+            and plan.state is opt.state
+            and plan.n_state == len(opt.state)
+            and plan.groups_key == groups_key
+            and (
+                plan.slots is None
+                or all(map(operator.is_, map(_MOMENTUM_OF, plan.slots), plan.bufs))
+            )
+        ):
+            return plan.entries
+        entries = _fusable_sgd(opt, params)
+        bufs = slots = None
+        if entries is not None and opt.state and not any(first for _, _, first in entries) and any(
+            sgd.momentum != 0.0 for _, sgd, _ in entries
+        ):
+            try:
+                slots = [opt.state[p] for p in self._param_objs]
+                bufs = [slot["momentum_buffer"] for slot in slots]
+            except KeyError:
+                slots = bufs = None
+        self._plan = _SgdPlan(entries, opt.state, len(opt.state), groups_key, bufs, slots)
+        if entries is None:
+            # the outer optimizer runs its own step(): buffers set aside for a fused one are
+            # not going to be used
+            self._placed_momentum = None
+        return entries
 
     def _momentum_buffers(self, idx: Sequence[int], first: bool) -> List[torch.Tensor]:
         """The outer SGD's momentum buffers; on the first step fresh tensors that are
         not yet part of the optimizer state (see ``_attach_momentum``)."""
-        live = [p for p in self._model.parameters()]
+        live = self._param_objs
+        placed = self._placed_momentum
         if first:
-            if self._placed_momentum is not None and all(
-                self._placed_momentum[i].shape == live[i].shape
-                and self._placed_momentum[i].dtype == live[i].dtype for i in idx
+            if placed is not None and all(
+                placed[i] is not None
+                and placed[i].shape == live[i].shape
+                and placed[i].dtype == live[i].dtype for i in idx
             ):
-                return [self._placed_momentum[i] for i in idx]
+                return [placed[i] for i in idx]
             key = "momentum/" + ",".join(map(str, idx[:4])) + f"/{len(idx)}"
             return self._flat_like(key, [live[i].data for i in idx])[1]
-        bufs = [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
-        placed = self._placed_momentum
-        if placed is not None and len(idx) == len(live) and all(
-            b.data_ptr() != placed[i].data_ptr() for b, i in zip(bufs, idx)
-        ):
-            # the optimizer state was replaced (a load_state_dict after healing): the buffers
-            # allocated for it at construction are not in use any more
-            self._placed_momentum = None
+        plan = self._plan
+        if plan is not None and plan.bufs is not None:
+            bufs = [plan.bufs[i] for i in idx]
+        else:
+            bufs = [self._outer_optimizer.state[live[i]]["momentum_buffer"] for i in idx]
+        if placed is not None:
+            # where the optimizer state was replaced (a load_state_dict after healing) the
+            # buffer set aside for it at construction is not in use any more: let it go
+            for b, i in zip(bufs, idx):
+                if placed[i] is not None and b.data_ptr() != placed[i].data_ptr():
+                    placed[i] = None
+            if all(t is None for t in placed):
+                self._placed_momentum = None
         return bufs
 
     def _attach_momentum(self, idx: Sequence[int], bufs: Sequence[torch.Tensor]) -> None:
         """After a committed first step the buffers become optimizer state, exactly where
         torch.optim.SGD keeps them."""
-        live = [p for p in self._model.parameters()]
+        live = self._param_objs
         for i, buf in zip(idx, bufs):
             self._outer_optimizer.state[live[i]]["momentum_buffer"] = buf
+        self._plan = None  # the next sync is a steady-state step
 
     def _outer_step(
         self,
@@ -522,13 +691,15 @@ class DiLoCo(LocalSGD):
         """Pseudo-gradients, their average over the replicas, restore, and (on commit)
         the outer step plus backup refresh (torchft/local_sgd.py:205-225)."""
         _, params, backups = self._named()
-        if not self._on_device(params, backups):
+        bound = self._bound
+        if not (bound.on_device if bound is not None and bound.params is params
+                else self._on_device(params, backups)):
             raise RuntimeError(
                 "DiLoCo needs parameters and backup on one GPU (the kernels have no CPU path); "
                 "construct it with backup_device=None or the parameters' device"
             )
-        live = list(self._model.parameters())
-        plan = _fusable_sgd(self._outer_optimizer, params)
+        live = self._param_objs
+        plan = self._sgd_plan(params)
         fused = self._fused(params, backups)
 
         if fused and plan is not None and self._manager.reduction_fails_only_at_launch():
@@ -591,35 +762,51 @@ class DiLoCo(LocalSGD):
     ) -> None:
         """The reduction is local and cannot fail once launched, so the commit decision
         can be taken first and the whole sync becomes one launch per parameter group:
-        either the fully fused step, or (no commit) a plain restore."""
+        either the fully fused step, or (no commit) a plain restore.  The prepared launches
+        (tensor lists and their validated table) are kept for as long as the parameters,
+        the backups, the plan and the peers' buffers are those of the previous sync."""
         manager = self._manager
         manager.wait_quorum()
         launches = []
+        mask = 0
         if manager.errored() is None:
             try:
-                replicas, mask = manager.replica_columns(params)
-                for gi, (idx, sgd, first) in enumerate(plan):
-                    bufs = self._momentum_buffers(idx, first) if sgd.momentum != 0.0 else None
-                    cols = dict(
-                        params=[params[i] for i in idx],
-                        backups=[backups[i] for i in idx],
-                        bufs=bufs,
-                        replicas=[[rep[i] for i in idx] for rep in replicas],
-                    )
-                    key = f"fused/{gi}"
-                    # built (and validated) before the vote: after it only the launch is left
-                    table = ops.diloco_outer_table(
-                        cols["params"], cols["backups"], bufs, cols["replicas"],
-                        table=self._tables.get(key),
-                    )
-                    launches.append((key, idx, cols, sgd, first, mask, table))
+                generation = self._generation
+                replicas, mask = manager.replica_columns(params, identity=(id(self), generation))
+                kept = self._launches.get("fused")
+                if (
+                    kept is not None
+                    and kept[0] == generation
+                    and kept[1] is replicas
+                    and kept[2] is plan
+                ):
+                    launches = kept[3]
+                else:
+                    for gi, (idx, sgd, first) in enumerate(plan):
+                        bufs = self._momentum_buffers(idx, first) if sgd.momentum != 0.0 else None
+                        cols = dict(
+                            params=[params[i] for i in idx],
+                            backups=[backups[i] for i in idx],
+                            bufs=bufs,
+                            replicas=[[rep[i] for i in idx] for rep in replicas],
+                        )
+                        key = f"fused/{gi}"
+                        # built (and validated) before the vote: after it only the launch is left
+                        table = ops.diloco_outer_table(
+                            cols["params"], cols["backups"], bufs, cols["replicas"],
+                            table=self._tables.get(key),
+                        )
+                        launches.append((key, idx, cols, sgd, first, table))
+                    if not any(first for _, _, first in plan):
+                        # a first step is prepared once only (its buffers become state)
+                        self._launches["fused"] = (generation, replicas, plan, launches)
             except Exception as e:  # same latch as Manager.allreduce
                 logger.exception("got exception preparing the fused sync -- skipping: %s", e)
                 manager.report_error(e)
                 launches = []
         if manager.should_commit():
             assert launches or not params, "a replica that failed to prepare cannot have voted to commit"
-            for key, idx, cols, sgd, first, mask, table in launches:
+            for key, idx, cols, sgd, first, table in launches:
                 self._tables[key] = ops.mt_diloco_outer(
                     cols["params"], cols["backups"], cols["bufs"], cols["replicas"], sgd, first,
                     mask, manager.num_participants(), table=table, table_is_current=True,
@@ -632,7 +819,7 @@ class DiLoCo(LocalSGD):
     def _average_grads(self) -> None:
         """One ``manager.allreduce`` per pseudo-gradient (torchft/local_sgd.py:227-239)."""
         works = []
-        for p in self._model.parameters():
+        for p in self._param_objs:
             assert p.grad is not None
             works.append(self._manager.allreduce(p.grad))
         for work in works:

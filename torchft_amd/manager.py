@@ -236,6 +236,7 @@ class Manager(Generic[T]):
         self._participating_rank: Optional[int] = None
         self._participating_world_size = 0
         self._tables: Dict[str, TensorTable] = {}
+        self._columns: Optional[tuple] = None  # replica_columns' previous answer and its key
 
     # ------------------------------------------------------------------ state
     def set_state_dict_fns(
@@ -546,13 +547,34 @@ class Manager(Generic[T]):
             self.report_error(e)
             return _done_future(grads)
 
-    def replica_columns(self, tensors: Sequence[torch.Tensor]):
-        """([replica][tensor] buffers in rank order, participation mask) for a tensor list."""
-        per_tensor = [self._pg.ordered(t, self.is_participating()) for t in tensors]
+    def replica_columns(self, tensors: Sequence[torch.Tensor], identity: object = None):
+        """([replica][tensor] buffers in rank order, participation mask) for a tensor list.
+
+        ``identity``: a hashable value by which the caller vouches for ``tensors`` (the same
+        value means the same tensors at the same addresses).  With it, and with a process
+        group whose peer buffers only change when it says so (``peers_generation``), the
+        columns of the previous call are returned as the very same list objects instead of
+        looking every tensor's peers up again; callers recognise an unchanged answer by
+        ``is``."""
+        participating = self.is_participating()
+        generation = None
+        if identity is not None:
+            peers_generation = getattr(self._pg, "peers_generation", None)
+            generation = peers_generation() if peers_generation is not None else None
+        if generation is not None:
+            key = (identity, generation, participating, len(tensors))
+            kept = self._columns
+            if kept is not None and kept[0] == key:
+                return kept[1], kept[2]
+        per_tensor = [self._pg.ordered(t, participating) for t in tensors]
         if not per_tensor:
             return [], 0
         n_rep = len(per_tensor[0][0])
-        return [[pt[0][r] for pt in per_tensor] for r in range(n_rep)], per_tensor[0][1]
+        columns = [[pt[0][r] for pt in per_tensor] for r in range(n_rep)]
+        mask = per_tensor[0][1]
+        if generation is not None:
+            self._columns = (key, columns, mask)
+        return columns, mask
 
     def reduction_fails_only_at_launch(self) -> bool:
         return bool(getattr(self._pg, "fails_only_at_launch", False))

@@ -170,6 +170,7 @@ class ProcessGroupLocalReplicas(ProcessGroup):
         world_size: int = 1,
         peer_lookup: Optional[PeerLookup] = None,
         peer_participating: Optional[Sequence[bool]] = None,
+        peers_are_stable: bool = False,
     ) -> None:
         super().__init__(rank, world_size)
         if not 0 <= rank < world_size:
@@ -179,6 +180,8 @@ class ProcessGroupLocalReplicas(ProcessGroup):
         self._rank = rank
         self._world = world_size
         self._lookup = peer_lookup
+        self._lookup_is_stable = peers_are_stable
+        self._generation = 0
         self._registry: Dict[Tuple[int, int], List[torch.Tensor]] = {}
         self._peer_participating = list(
             peer_participating if peer_participating is not None else [True] * (world_size - 1)
@@ -205,19 +208,39 @@ class ProcessGroupLocalReplicas(ProcessGroup):
         return "torchft-local-replicas"
 
     # -- peers -------------------------------------------------------------
-    def set_peer_lookup(self, peer_lookup: Optional[PeerLookup]) -> None:
+    def set_peer_lookup(self, peer_lookup: Optional[PeerLookup], peers_are_stable: bool = False) -> None:
         self._lookup = peer_lookup
+        self._lookup_is_stable = peers_are_stable
+        self._generation += 1
 
     def set_peer_participating(self, flags: Sequence[bool]) -> None:
         if len(flags) != self._world - 1:
             raise ValueError("peer_participating needs one entry per peer")
         self._peer_participating = list(flags)
+        self._generation += 1
+
+    def invalidate_peers(self) -> None:
+        """Says that the peers' buffers may have moved (for lookups declared stable)."""
+        self._generation += 1
+
+    def peers_generation(self) -> Optional[int]:
+        """A counter that changes whenever the answer of :meth:`ordered` may change for a
+        tensor that has not moved, or None if that cannot be known: a ``peer_lookup``
+        callback may return different buffers from one call to the next unless it was
+        declared stable (``peers_are_stable=True``: it returns the same buffers for the
+        same tensor until ``invalidate_peers()`` / ``set_peer_lookup()``).  Registered peers
+        (``register_peers``) only change through this object.  Callers that hold a whole
+        model's peer columns use it to skip one lookup per tensor per sync."""
+        if self._lookup is not None and not self._lookup_is_stable:
+            return None
+        return self._generation
 
     def register_peers(self, tensor: torch.Tensor, peers: Sequence[torch.Tensor]) -> None:
         """Declares the peers' buffers for ``tensor`` (matched by address and size)."""
         if len(peers) != self._world - 1:
             raise ValueError(f"{len(peers)} peer tensors for a world of {self._world}")
         self._registry[(tensor.data_ptr(), tensor.numel())] = list(peers)
+        self._generation += 1
 
     def peers_of(self, tensor: torch.Tensor) -> List[torch.Tensor]:
         if self._world == 1:
