@@ -40,7 +40,8 @@ HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
              "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
              "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b",
-             "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b", "localsgd_llama3_8b_api"]
+             "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b", "localsgd_llama3_8b_api",
+             "ddp_hook_llama3_8b", "diloco_gpt2_small_api"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -50,6 +51,8 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=WORKLOADS, default=WORKLOADS[0])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-api", action="store_true",
+                    help="headline workload: leave out the sub-record measured through DiLoCo.sync()")
     ap.add_argument("--cpu-layers", type=int, default=8,
                     help="decoder layers in the CPU baseline's slice of the Llama workload")
     ap.add_argument("--cpu-steps", type=int, default=4)
@@ -151,6 +154,52 @@ def base_line(args, metric: str, value: float, unit: str, ms_per_step: float, dt
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": config,
     }
+
+
+class CheckerReplay:
+    """Output check of a timed DiLoCo run: the initial state of a few whole tensors is kept on
+    the host, the CPU checker replays as many outer steps as the GPU ran, and parameters,
+    backup and momentum must come out bit for bit.  ``in_place``: replica 0 is the live
+    parameter tensor (what ``DiLoCo.sync()`` does), so every step reads the previous step's
+    parameters."""
+
+    MAX_ELEMS = 5_000_000
+
+    def __init__(self, backup, bufs, replicas, in_place: bool, want: int = 3) -> None:
+        small = [i for i, t in enumerate(backup) if t.numel() <= self.MAX_ELEMS]
+        picks = sorted({small[0], small[len(small) // 2], small[-1]}) if small else []
+        biggest_small = max(small, key=lambda i: backup[i].numel()) if small else None
+        if biggest_small is not None:
+            picks = sorted(set(picks[:want - 1]) | {biggest_small})
+        self.picks = picks
+        self.in_place = in_place
+        self.backup = [backup[i].detach().cpu().clone() for i in picks]
+        self.bufs = None if bufs is None else [bufs[i].detach().cpu().clone() for i in picks]
+        self.replicas = [[rep[i].detach().cpu().clone() for i in picks] for rep in replicas]
+
+    def check(self, steps: int, params, backup, bufs, dtype: torch.dtype) -> str:
+        from oracle import replica_sync as O
+
+        if not self.picks:
+            return "skipped: no tensor small enough to replay on the host"
+        n = len(self.replicas)
+        acc = None if dtype == torch.float32 else torch.float32
+        reps, b, m = self.replicas, self.backup, self.bufs
+        for _ in range(steps):
+            out = O.diloco_perform_sync(reps, b, m, [True] * n, n, True, lr=LR, momentum=MOMENTUM,
+                                        nesterov=True, accumulate_dtype=acc)
+            b, m = out["backup"], out["momentum"]
+            if self.in_place:
+                reps = [out["params"], *reps[1:]]
+        for k, i in enumerate(self.picks):
+            for got, want, what in ((params[i], out["params"][k], "parameters"),
+                                    (backup[i], b[k], "backup"), (bufs[i], m[k], "momentum")):
+                if not torch.equal(got.detach().cpu().view(torch.uint8), want.view(torch.uint8)):
+                    raise RuntimeError(f"output check failed: {what} of tensor {i} differ from the "
+                                       f"CPU checker after {steps} steps")
+        elems = sum(t.numel() for t in self.backup)
+        return (f"parameters, backup and momentum of tensors {self.picks} ({elems} elements) equal the CPU "
+                f"checker's bit for bit after {steps} outer steps")
 
 
 # ---------------------------------------------------------------------------
@@ -297,6 +346,7 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         pristine = ([t.clone() for t in wl.backup], [t.clone() for t in bufs])
     done = [0]
     reseeds = [0]
+    replay = None if need_reseed else CheckerReplay(wl.backup, bufs, wl.replicas, in_place="alias_p" in layout)
 
     def step() -> None:
         if pristine is not None and done[0] and done[0] % RESEED == 0:
@@ -311,6 +361,8 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
         same = torch.equal(params[probe].view(torch.uint8), wl.backup[probe].view(torch.uint8))
         if not same or not torch.isfinite(params[probe]).all():
             raise RuntimeError("output check failed: parameters are not finite or differ from the backup")
+    checked = ("skipped: the state is re-seeded inside the timed region" if replay is None
+               else replay.check(done[0], params, wl.backup, bufs, dtype))
 
     n_params = wl.n_params
     # read N replicas, backup, momentum; write momentum, parameters, backup
@@ -324,7 +376,7 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
          "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
          "allocation": ("every tensor is a contiguous view carved out of one device allocation"
                         if args.arena else "one device allocation per tensor"),
-         "layout": layout, "model_copies": args.model_copies})
+         "layout": layout, "model_copies": args.model_copies, "output_check": checked})
     out["roofline"] = roofline(algo_bytes, kernel_ms,
                                f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<{n_rep}>>",
                                workload="" if args.model_copies > 1 else
@@ -343,16 +395,20 @@ def bench_diloco(args, which: str) -> Dict[str, object]:
     return out
 
 
-def bench_diloco_api(args) -> Dict[str, object]:
+def bench_diloco_api(args, which: str = "llama3_8b") -> Dict[str, object]:
     """The same step driven through the torchft-shaped API: ``DiLoCo.sync()`` on a module
-    with the 291 Llama-3-8B parameters, this package's Manager on a local replica group of
-    2; the timed step includes all host work (quorum, commit vote, table checks)."""
+    with the model's parameters, this package's Manager on a local replica group; the timed
+    step includes all host work (quorum, commit vote, validation of the kept launch).  The
+    parameters are replica 0 and are updated in place, as the reference's ``p.data`` are."""
     from torch import nn
 
     from torchft_amd import DiLoCo, Manager, ProcessGroupLocalReplicas, StaticQuorum, workloads
 
     dev = torch.device("cuda", 0)
-    shapes = workloads.llama3_8b_shapes()
+    if which == "llama3_8b":
+        shapes, n_rep = workloads.llama3_8b_shapes(), 2
+    else:
+        shapes, n_rep = workloads.gpt2_small_shapes(), 4
     dtype = torch.bfloat16 if args.storage_dtype == "bf16" else torch.float32
     esize = 2 if dtype == torch.bfloat16 else 4
 
@@ -363,33 +419,79 @@ def bench_diloco_api(args) -> Dict[str, object]:
                 [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev, dtype)])
 
     model = Bag()
-    peer = workloads.drifted_replica([p.data for p in model.parameters()], 1e-3, 1001)
+    live = [p.data for p in model.parameters()]
+    peers = [workloads.drifted_replica(live, 1e-3, 1001 + r) for r in range(n_rep - 1)]
     index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
-    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+    # the peers' buffers stay where they are for the whole run: the group may say so, and a
+    # sync then does not ask for every tensor's peers again
+    pg = ProcessGroupLocalReplicas(0, n_rep, peer_lookup=lambda t: [pr[index[t.data_ptr()]] for pr in peers],
+                                   peers_are_stable=True)
     manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
-                      quorum_client=StaticQuorum(0, 2))
+                      quorum_client=StaticQuorum(0, n_rep))
     inner = torch.optim.SGD(model.parameters(), lr=0.1)
     outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
     n_params = sum(p.numel() for p in model.parameters())
     if args.steps + args.warmup > 60:
-        raise SystemExit("diloco_llama3_8b_api: at most 60 syncs in total (static peers make the "
+        raise SystemExit(f"diloco_{which}_api: at most 60 syncs in total (static peers make the "
                          "backup run away from them; see bench_diloco)")
+    host_ms, isolated_ms = [], []
     with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
+        backups = list(diloco._backup_parameters.values())
+        replay = CheckerReplay(backups, None, [live, *peers], in_place=True)
         diloco.sync()  # first step creates the momentum state
-        wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(diloco.sync)
+
+        def timed_sync() -> None:
+            t0 = time.perf_counter()
+            diloco.sync()
+            host_ms.append((time.perf_counter() - t0) * 1e3)
+
+        wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(timed_sync)
+        n_syncs = 1 + args.warmup + args.steps
+        if which != "llama3_8b":
+            # a sync as a training loop sees it: device idle before, result awaited after
+            for _ in range(10):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                diloco.sync()
+                torch.cuda.synchronize()
+                isolated_ms.append((time.perf_counter() - t0) * 1e3)
+            n_syncs += 10
+        bufs = [outer.state[p]["momentum_buffer"] for p in model.parameters()]
+        checked = replay.check(n_syncs, [p.data for p in model.parameters()], backups, bufs, dtype)
     manager.shutdown(wait=False)
-    out = base_line(args, HEADLINE_METRIC + " (through DiLoCo.sync())", n_params / (wall_ms * 1e-3),
+    metric = HEADLINE_METRIC if which == "llama3_8b" else "outer-sync params/sec, GPT-2-small DiLoCo"
+    out = base_line(args, metric + " (through DiLoCo.sync())", n_params / (wall_ms * 1e-3),
                     "params/s", wall_ms, "f32",
-                    {"workload": "DiLoCo.sync() on a module with the 291 Llama-3-8B "
+                    {"workload": f"DiLoCo.sync() on a module with the {len(shapes)} {which} "
                                  f"{'fp32' if esize == 4 else 'bf16'} parameters, "
-                                 "Manager + ProcessGroupLocalReplicas(world 2), outer torch.optim.SGD "
+                                 f"Manager + ProcessGroupLocalReplicas(world {n_rep}), outer torch.optim.SGD "
                                  "Nesterov; parameters updated in place (the live parameters are "
-                                 "replica 0)",
-                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
-    out["roofline"] = roofline(n_params * 7 * esize, kernel_ms,
-                               f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<2>>")
+                                 "replica 0); backup and momentum allocated by the library",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep,
+                     "output_check": checked})
+    out["roofline"] = roofline(n_params * (n_rep + 5) * esize, kernel_ms,
+                               f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<{n_rep}>>")
     out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
+    timed = host_ms[args.warmup:]
+    out["host_ms_per_sync"] = sum(timed) / len(timed)
+    if isolated_ms:
+        out["isolated_sync_ms"] = sum(isolated_ms) / len(isolated_ms)
     return out
+
+
+def api_record(line: Dict[str, object]) -> Dict[str, object]:
+    """The drop-in seat's figures as a sub-record of the headline line."""
+    roof = line["roofline"]
+    return {
+        "workload": line["config"]["workload"],
+        "ms_per_step": line["ms_per_step"],
+        "params_per_s": line["value"],
+        "kernel_ms_per_step": roof["kernel_ms_per_step"],
+        "achieved_GBs": roof["achieved"],
+        "frac": roof["frac"],
+        "host_ms_per_sync": line["host_ms_per_sync"],
+        "output_check": line["config"]["output_check"],
+    }
 
 
 def bench_localsgd_api(args) -> Dict[str, object]:
@@ -764,6 +866,164 @@ def bench_ddp_buckets(args, form: str = "hook_order") -> Dict[str, object]:
     return out
 
 
+def bench_ddp_hook(args) -> Dict[str, object]:
+    """Gradient-bucket averaging through the reference's own seat (torchft/ddp.py:47-71): a module
+    with the 291 Llama-3-8B bf16 parameters in ``DistributedDataParallel(manager, module,
+    gradient_as_bucket_view=True)``; torch's Reducer owns the flat buckets and calls the
+    communication hook as each fills during a real backward; the hook is
+    ``manager.allreduce(bucket.buffer())`` on a local replica group of 4 of which one is a spare
+    (3 participate).  Everything runs on one stream, so GPU time is additive: the same backward
+    is timed with the averaging hook and with ``manager.allreduce`` replaced by a stand-in that
+    only returns the bucket, and HIP events around every ``manager.allreduce`` call give the
+    averaging kernels' own time."""
+    from torch import nn
+
+    from oracle import replica_sync as O
+    from torchft_amd import (DistributedDataParallel, Manager, ProcessGroupLocalReplicas, StaticQuorum,
+                             WorldSizeMode, workloads)
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+    n_rep, n_active = 4, 3
+
+    class Bag(nn.Module):
+        """loss = sum_i <p_i, w_i>: the backward hands the Reducer dense bf16 gradients (= w_i)."""
+
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList(
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev, torch.bfloat16)])
+            self.ws = workloads.normal_tensors(shapes, 1e-2, workloads.SEED_GRAD, dev, torch.bfloat16)
+
+        def forward(self) -> torch.Tensor:
+            total = torch.zeros((), device=dev, dtype=torch.float32)
+            for p, w in zip(self.ps, self.ws):
+                total = total + (p * w).sum(dtype=torch.float32)
+            return total
+
+    model = Bag()
+    n_elems = sum(p.numel() for p in model.parameters())
+    peer_bufs: Dict[int, List[torch.Tensor]] = {}
+    gen = torch.Generator(device=dev).manual_seed(workloads.SEED_GRAD + 1)
+
+    def peers_of(flat: torch.Tensor) -> List[torch.Tensor]:
+        # the peers' copies of this bucket: drawn the first time the bucket is seen, then kept
+        key = flat.data_ptr()
+        if key not in peer_bufs:
+            peer_bufs[key] = [
+                torch.empty(flat.numel(), dtype=torch.float32, device=dev).normal_(0.0, 1e-2, generator=gen)
+                .to(flat.dtype) for _ in range(n_rep - 1)]
+        return peer_bufs[key]
+
+    pg = ProcessGroupLocalReplicas(0, n_rep, peer_lookup=peers_of, peers_are_stable=True,
+                                   peer_participating=[True, True, False])
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=n_active,
+                      world_size_mode=WorldSizeMode.FIXED_WITH_SPARES, quorum_client=StaticQuorum(0, n_rep))
+    ddp = DistributedDataParallel(manager, model, gradient_as_bucket_view=True)
+    allreduce = manager.allreduce
+    mode = {"average": True, "record": False}
+    host_us: List[float] = []
+    spans: List[Tuple[torch.cuda.Event, torch.cuda.Event]] = []
+    buckets: Dict[int, torch.Tensor] = {}
+
+    def instrumented(tensor: torch.Tensor):
+        # sits one call below the hook itself (DistributedDataParallel._comm_hook stays in
+        # its seat: a Reducer takes only one hook for its lifetime)
+        if not mode["average"]:
+            fut: torch.futures.Future = torch.futures.Future()
+            fut.set_result(tensor)
+            return fut
+        buckets.setdefault(tensor.data_ptr(), tensor)
+        if not mode["record"]:
+            return allreduce(tensor)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        t0 = time.perf_counter()
+        fut = allreduce(tensor)
+        host_us.append((time.perf_counter() - t0) * 1e6)
+        b.record()
+        spans.append((a, b))
+        return fut
+
+    manager.allreduce = instrumented
+
+    def backward(average: bool, record: bool = False) -> Tuple[float, float]:
+        mode["average"], mode["record"] = average, record
+        for p in model.parameters():
+            p.grad = None
+        manager.start_quorum()
+        loss = ddp()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        a.record()
+        loss.backward()
+        b.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        if not manager.should_commit():
+            raise RuntimeError(f"the step did not commit: {manager.errored()!r}")
+        return a.elapsed_time(b), wall
+
+    for _ in range(max(args.warmup, 2)):
+        backward(True)
+        backward(False)
+    with_hook, without, kernels, walls = [], [], [], []
+    for _ in range(args.steps):
+        host_us.clear()
+        spans.clear()
+        gpu_ms, wall_ms = backward(True, record=True)
+        with_hook.append(gpu_ms)
+        walls.append(wall_ms)
+        kernels.append(sum(a.elapsed_time(b) for a, b in spans))
+        n_hooks, host_per_hook = len(spans), sum(host_us) / max(len(host_us), 1)
+        without.append(backward(False)[0])
+    mean = lambda xs: sum(xs) / len(xs)
+
+    # spot check of the last averaged backward against the checker: whole gradients of a few
+    # parameters, located inside their bucket by address
+    backward(True)
+    params = list(model.parameters())
+    small = [i for i, p in enumerate(params) if p.numel() <= 5_000_000]
+    picks = sorted({small[0], small[len(small) // 2], small[-1], max(small, key=lambda i: params[i].numel())})
+    for i in picks:
+        g = params[i].grad
+        home = next(((ptr, flat) for ptr, flat in buckets.items()
+                     if ptr <= g.data_ptr() < ptr + flat.numel() * 2), None)
+        if home is None:
+            raise RuntimeError(f"output check failed: gradient {i} is not a view of a bucket")
+        off = (g.data_ptr() - home[0]) // 2
+        contributions = [model.ws[i].reshape(-1).cpu()] + [
+            pb[off:off + g.numel()].cpu() for pb in peer_bufs[home[0]]]
+        want = O.manager_allreduce_(contributions, [True, True, True, False], n_active, torch.float32)
+        if not torch.equal(g.reshape(-1).cpu().view(torch.int16), want.view(torch.int16)):
+            raise RuntimeError(f"output check failed: gradient {i} differs from the CPU checker")
+    manager.shutdown(wait=False)
+
+    hook_ms = mean(with_hook) - mean(without)
+    out = base_line(args, "DDP gradient-bucket average elements/sec through the comm hook, Llama-3-8B bf16",
+                    n_elems / (mean(kernels) * 1e-3), "elements/s", mean(kernels), "bf16 storage, f32 accumulate",
+                    {"workload": f"torch DistributedDataParallel(gradient_as_bucket_view=True) over the {len(shapes)} "
+                                 f"Llama-3-8B bf16 parameters ({n_elems} elements), {n_hooks} buckets, comm hook = "
+                                 "manager.allreduce(bucket.buffer()) on ProcessGroupLocalReplicas(world 4, one spare, "
+                                 "3 participate); one step = one real backward; ms_per_step is the sum of the "
+                                 "averaging kernels' time (HIP events around each manager.allreduce call)",
+                     "n_buckets": n_hooks, "n_elements": n_elems,
+                     "output_check": f"gradients {picks} equal the CPU checker's bucket average bit for bit"})
+    out["roofline"] = roofline(n_elems * 2 * (n_active + 1), mean(kernels),
+                               "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>, FlatLocator>", n_hooks)
+    out["hook_seat"] = {
+        "backward_gpu_ms_with_averaging_hook": mean(with_hook),
+        "backward_gpu_ms_with_pass_through_hook": mean(without),
+        "difference_ms": hook_ms,
+        "frac_of_peak_by_difference": n_elems * 2 * (n_active + 1) / (hook_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "backward_wall_ms_with_averaging_hook": mean(walls),
+        "host_us_per_hook": host_per_hook,
+        "hooks_per_backward": n_hooks,
+    }
+    return out
+
+
 def bench_checkpoint(args) -> Dict[str, object]:
     from torchft_amd import state_pack, workloads
 
@@ -926,6 +1186,16 @@ def main() -> int:
         torch.cuda.empty_cache()
     if args.workload == "diloco_llama3_8b":
         out = bench_diloco(args, "llama3_8b")
+        if not args.no_api and args.model_copies == 1 and not args.arena:
+            # the same step through the reference's own seat, in the same process: the
+            # kernel-level tensors are gone by now (they were locals of bench_diloco)
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            out["api"] = api_record(bench_diloco_api(args))
+    elif args.workload == "diloco_gpt2_small_api":
+        out = bench_diloco_api(args, "gpt2_small")
+    elif args.workload == "ddp_hook_llama3_8b":
+        out = bench_ddp_hook(args)
     elif args.workload == "diloco_gpt2_small":
         out = bench_diloco(args, "gpt2_small")
     elif args.workload == "ddp_buckets_llama3_8b":

@@ -47,7 +47,8 @@
  *   - the sum is divided (IEEE divide, not reciprocal multiply) by
  *     num_participants, which may differ from popcount(participate_mask);
  *   - bf16 and fp16 inputs are widened to fp32, accumulated and divided in fp32,
- *     and rounded to nearest-even once on store.
+ *     and rounded to nearest-even once on store;
+ *   - fp64 inputs (replica average only) are accumulated and divided in fp64.
  */
 #ifndef TORCHFT_AMD_H_
 #define TORCHFT_AMD_H_
@@ -58,7 +59,7 @@
 extern "C" {
 #endif
 
-#define TFT_ABI_VERSION 4
+#define TFT_ABI_VERSION 5
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
 #define TFT_MIN_CHUNK_ELEMS 8192u
 #define TFT_NOALLOC_MAX_TENSORS 4096u /* rows of the built-in table of the allocation-free entry */
@@ -70,7 +71,9 @@ typedef enum tft_status {
   TFT_ERR_LAUNCH = -3
 } tft_status;
 
-typedef enum tft_dtype { TFT_F32 = 0, TFT_BF16 = 1, TFT_F16 = 2 } tft_dtype;
+/* TFT_F64 is accepted by the replica average (tft_reduce_avg, tft_mt_reduce_avg) only:
+ * Manager.allreduce is dtype-generic in the reference (torchft/manager.py:267-287). */
+typedef enum tft_dtype { TFT_F32 = 0, TFT_BF16 = 1, TFT_F16 = 2, TFT_F64 = 3 } tft_dtype;
 
 /* Host struct describing one multi-tensor table (the arrays live on the device). */
 typedef struct tft_mt_table {

@@ -56,7 +56,11 @@ def test_abi_version_and_constants():
     assert _native.ABI_VERSION == lib.tft_abi_version()
     assert _native.MAX_REPLICAS == int(re.search(r"#define TFT_MAX_REPLICAS (\d+)", text).group(1))
     assert _native.MIN_CHUNK_ELEMS == int(re.search(r"#define TFT_MIN_CHUNK_ELEMS (\d+)u", text).group(1))
-    for code in (_native.TFT_F32, _native.TFT_BF16, -1):
+    dtypes = re.search(r"typedef enum tft_dtype \{([^}]*)\}", text).group(1)
+    declared = {k.strip(): int(v) for k, v in (item.split("=") for item in dtypes.split(","))}
+    assert declared == {"TFT_F32": _native.TFT_F32, "TFT_BF16": _native.TFT_BF16,
+                        "TFT_F16": _native.TFT_F16, "TFT_F64": _native.TFT_F64}
+    for code in (_native.TFT_F32, _native.TFT_BF16, _native.TFT_F64, -1):
         chunk = lib.tft_default_chunk_elems(code)
         assert chunk >= _native.MIN_CHUNK_ELEMS and chunk & (chunk - 1) == 0
 
@@ -118,6 +122,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.tft_mt_diloco_outer(ctypes.byref(table), 3, 7, 3, 0, ctypes.byref(sgd), None) == -1
     assert b"columns" in lib.tft_last_error()
     assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, 9, ctypes.byref(sgd), None) == -2  # dtype
+    # fp64 is the replica average's alone
+    assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, _native.TFT_F64, ctypes.byref(sgd), None) == -2
+    assert b"replica average only" in lib.tft_last_error()
+    assert lib.tft_reduce_avg(None, None, 1, 1, 1, 0, _native.TFT_F64, None) == 0
     # an empty table is a successful no-op
     assert lib.tft_mt_diloco_outer(ctypes.byref(table), 2, 3, 2, 0, ctypes.byref(sgd), None) == 0
 

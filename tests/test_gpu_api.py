@@ -159,6 +159,80 @@ def test_manager_error_latch_on_gpu(device):
     m.shutdown(wait=False)
 
 
+def test_manager_allreduce_is_dtype_generic_and_never_raises(device):
+    """torchft/manager.py:242-303 reduces whatever floating tensor it is given and never raises.
+    fp64 runs in fp64 (oracle bits); a tensor the kernels cannot take (integer, not contiguous,
+    on the host) is latched like any failed all-reduce: the future completes with the tensor
+    untouched, later calls are no-ops, the step does not commit, the next quorum clears it."""
+    n = 100_003
+    g = torch.Generator().manual_seed(3)
+    xs = [torch.randn(n, generator=g, dtype=torch.float64) for _ in range(3)]
+    dev = [x.to(device) for x in xs]
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=3, peer_participating=[True, False])
+    pg.register_peers(dev[0], dev[1:])
+    m = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                quorum_client=StaticQuorum(0, 3))
+    m.start_quorum()
+    assert m.allreduce(dev[0]).wait() is dev[0]
+    assert m.errored() is None
+    assert_bits_equal(dev[0], O.manager_allreduce_(xs, [True, True, False], 3))
+    assert m.should_commit()
+
+    for make, kind in (
+        (lambda: torch.arange(8, device=device), TypeError),                   # integer
+        (lambda: torch.ones(4, 6, device=device).t(), ValueError),             # not contiguous
+        (lambda: torch.ones(8), RuntimeError),                                 # host memory
+    ):
+        m.start_quorum()
+        t = make()
+        before = t.clone()
+        fut = m.allreduce(t)          # must not raise
+        assert fut.wait() is t
+        assert isinstance(m.errored(), kind), m.errored()
+        assert torch.equal(t, before)
+        other = torch.ones(8, device=device)
+        assert m.allreduce(other).wait() is other  # a no-op until the next quorum
+        assert_bits_equal(other, torch.ones(8))
+        assert not m.should_commit()
+    m.start_quorum()
+    assert m.errored() is None
+    m.shutdown(wait=False)
+
+
+def test_localsgd_on_fp64_parameters(device):
+    """LocalSGD is dtype-generic in the reference (torchft/local_sgd.py:97-174); fp64 parameters
+    are averaged in fp64 and backed up byte for byte."""
+    torch.manual_seed(0)
+    model = Tiny().to(device=device, dtype=torch.float64)
+    peers, lookup = peer_world(model, 2)
+    for q in peers[0].parameters():
+        q.data.add_(1e-9)  # below fp32 resolution of the values
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    optimizer = optim.SGD(model.parameters(), lr=1e-3)
+    with LocalSGD(manager, model, optimizer, sync_every=10 ** 9) as lsgd:
+        backup0 = cpu(lsgd._backup_parameters.values())
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(3e-9)
+        local = cpu(p.data for p in model.parameters())
+        want = O.localsgd_perform_sync([local, cpu(q.data for q in peers[0].parameters())],
+                                       backup0, [True, True], 2, True)
+        lsgd.sync()
+        for p, w, b in zip(model.parameters(), want["params"], lsgd._backup_parameters.values()):
+            assert p.dtype == torch.float64
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(b, w)
+    # DiLoCo's outer step is fp32 arithmetic: fp64 parameters are refused at construction
+    manager2 = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                       use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    with pytest.raises(TypeError, match="float64"):
+        DiLoCo(manager2, model, optimizer, optim.SGD(model.parameters(), lr=0.7), sync_every=2)
+    manager.shutdown(wait=False)
+    manager2.shutdown(wait=False)
+
+
 # ---------------------------------------------------------------------------
 # LocalSGD / DiLoCo
 # ---------------------------------------------------------------------------

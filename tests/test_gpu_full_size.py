@@ -109,6 +109,71 @@ def test_diloco_llama3_8b_full_size_bf16_in_place(device):
         assert_bits_equal(take(wl.replicas[1][i], spans[i]), peer_before[i])
 
 
+def test_diloco_sync_llama3_8b_full_size_fp32_through_the_api(device):
+    """Config 4 through the reference's own seat: ``DiLoCo.sync()`` on a module with the 291
+    fp32 Llama-3-8B parameters, this package's Manager on a local replica group of 2, outer
+    ``torch.optim.SGD`` (Nesterov).  The parameters are replica 0 and are updated in place;
+    backup and momentum are the library's own (placed) buffers.  A first sync and two
+    steady-state syncs: windows of every tensor of the parameters, the backup and
+    ``outer_optimizer.state[p]["momentum_buffer"]`` against the checker, backup == parameters
+    everywhere, the peer untouched, ``id(param)`` and the inner optimizer's state intact."""
+    from torch import nn, optim
+
+    from torchft_amd import DiLoCo, Manager, ProcessGroupLocalReplicas, StaticQuorum
+
+    shapes = workloads.llama3_8b_shapes()
+
+    class Bag(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList(
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, workloads.SEED_BACKUP, device)])
+
+    model = Bag()
+    params = list(model.parameters())
+    assert sum(p.numel() for p in params) == 8_030_261_248
+    peer = workloads.drifted_replica([p.data for p in params], 1e-3, workloads.SEED_REPLICA + 1)
+    index = {p.data_ptr(): i for i, p in enumerate(params)}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]],
+                                   peers_are_stable=True)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(params, lr=0.1, momentum=0.5)
+    outer = optim.SGD(params, lr=0.7, momentum=0.9, nesterov=True)
+    ids = [id(p) for p in params]
+    gen = torch.Generator().manual_seed(17)
+    spans = [windows(p.numel(), gen) for p in params]
+    peer_before = [take(t, s) for t, s in zip(peer, spans)]
+    with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
+        backups = list(diloco._backup_parameters.values())
+        assert outer.state_dict()["state"] == {}
+        bufs_before = None
+        for step in range(3):
+            # the replica has drifted since the last sync (inner steps): here one known shift
+            with torch.no_grad():
+                torch._foreach_add_([p.data for p in params], 1e-3 * (step + 1))
+            local = [take(p.data, s) for p, s in zip(params, spans)]
+            before_b = [take(b, s) for b, s in zip(backups, spans)]
+            diloco.sync()
+            want = O.diloco_perform_sync([local, peer_before], before_b, bufs_before, [True, True], 2,
+                                         True, lr=0.7, momentum=0.9, nesterov=True)
+            for i, (name, _) in enumerate(shapes):
+                assert_bits_equal(take(params[i].data, spans[i]), want["params"][i], f"sync {step} {name}")
+                assert_bits_equal(take(backups[i], spans[i]), want["backup"][i], f"sync {step} backup {name}")
+                assert_bits_equal(take(outer.state[params[i]]["momentum_buffer"], spans[i]),
+                                  want["momentum"][i], f"sync {step} momentum {name}")
+            assert all(torch.equal(p.data, b) for p, b in zip(params, backups))
+            assert all(p.grad is None for p in params)
+            bufs_before = want["momentum"]
+        assert len(outer.state_dict()["state"]) == len(params)
+    assert manager.current_step() == 3
+    assert [id(p) for p in model.parameters()] == ids
+    assert list(diloco._backup_parameters.values())[0] is backups[0]
+    for i in range(len(shapes)):
+        assert_bits_equal(take(peer[i], spans[i]), peer_before[i])
+    manager.shutdown(wait=False)
+
+
 def test_ddp_buckets_llama3_8b_full_size(device):
     """bf16 gradients of Llama-3-8B, 162 buckets by torch's rule, 4 contributions of which
     3 participate, fp32 accumulation, result written over replica 0's gradients."""

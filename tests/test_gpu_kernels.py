@@ -66,6 +66,81 @@ def test_reduce_avg_in_place_and_misaligned(device, dtype):
     assert_bits_equal(out2, want2)
 
 
+# ---------------------------------------------------------------------------
+# fp64: the replica average is dtype-generic in the reference (torchft/manager.py:267-287)
+# ---------------------------------------------------------------------------
+
+def draw64(n, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, generator=g, dtype=torch.float64) * scale
+
+
+@pytest.mark.parametrize("n_replicas,mask,nump", [
+    (1, 0b1, 1), (1, 0b1, 5), (1, 0b0, 5), (2, 0b11, 2), (3, 0b101, 2), (4, 0b1011, 3),
+    (4, 0b1111, 4), (8, 0xFF, 8), (8, 0b10110101, 2), (0, 0, 3),
+])
+def test_reduce_avg_flat_fp64(device, n_replicas, mask, nump):
+    """fp64 buffers are summed and divided in fp64, exactly as torch does on the host: the
+    mantissa bits beyond fp32 must survive (values drawn in fp64, scaled apart)."""
+    for numel in SIZES:
+        reps = [draw64(numel, 10 * r + numel % 7, 10.0 ** (r % 3)) for r in range(n_replicas)]
+        if n_replicas:
+            want = O.manager_allreduce_(reps, mask_to_list(mask, n_replicas), nump)
+        else:
+            want = torch.zeros(numel, dtype=torch.float64)
+        out = torch.full((numel,), 7.0, dtype=torch.float64, device=device)
+        ops.reduce_avg_(out, [r.to(device) for r in reps], mask, nump)
+        assert_bits_equal(out, want, f"numel={numel}")
+    # not merely fp32 arithmetic widened: 1 + 2^-40 is not representable in fp32
+    a = torch.tensor([1.0, 3.0], dtype=torch.float64, device=device)
+    b = torch.tensor([2.0 ** -40, 2.0 ** -45], dtype=torch.float64, device=device)
+    out = torch.empty_like(a)
+    ops.reduce_avg_(out, [a, b], 0b11, 3)
+    assert_bits_equal(out, (torch.tensor([1.0 + 2.0 ** -40, 3.0 + 2.0 ** -45], dtype=torch.float64)) / 3)
+
+
+def test_reduce_avg_fp64_in_place_misaligned_and_multi_tensor(device):
+    numel = 70_001
+    reps = [draw64(numel + 1, 50 + r) for r in range(3)]
+    want = O.manager_allreduce_([r[1:] for r in reps], [True, True, True], 3)
+    dev = [r.to(device) for r in reps]
+    out = dev[1][1:]                      # 8 bytes past a 16-byte boundary, aliases replica 1
+    ops.reduce_avg_(out, [d[1:] for d in dev], 0b111, 3)
+    assert_bits_equal(out, want)
+    assert_bits_equal(dev[1][:1], reps[1][:1])
+    # columns misaligned differently from each other: the scalar path
+    dev2 = [r.to(device) for r in reps]
+    out2 = torch.empty(numel, dtype=torch.float64, device=device)
+    ops.reduce_avg_(out2, [dev2[0][1:], dev2[1][:-1], dev2[2][1:]], 0b110, 2)
+    want2 = O.manager_allreduce_([reps[0][1:], reps[1][:-1], reps[2][1:]], [False, True, True], 2)
+    assert_bits_equal(out2, want2)
+    # a table of ragged tensors, two outputs (LocalSGD: parameters and backup together)
+    sizes = [1, 0, 5, 1023, 1025, 40_000, 66_000, 131_073]
+    cols = [[draw64(n, 300 + 17 * r + i) for i, n in enumerate(sizes)] for r in range(2)]
+    dev_cols = [[t.to(device) for t in col] for col in cols]
+    p = dev_cols[0]                       # in place on replica 0
+    bkp = [torch.full_like(t, 5.0) for t in p]
+    ops.mt_reduce_avg([p, bkp], dev_cols, 0b11, 2)
+    for i, n in enumerate(sizes):
+        want = O.manager_allreduce_([cols[0][i], cols[1][i]], [True, True], 2)
+        assert_bits_equal(p[i], want, f"tensor {i} ({n})")
+        assert_bits_equal(bkp[i], want, f"backup {i} ({n})")
+
+
+def test_fp64_over_the_whole_encoding(device):
+    """Random bit patterns (denormals, infinities, NaNs, values next to overflow) through the
+    fp64 average: bit-equal wherever the checker has a number, NaN wherever it has a NaN."""
+    g = torch.Generator().manual_seed(11)
+    n = 300_000
+    reps = [torch.randint(-2 ** 63, 2 ** 63 - 1, (n,), generator=g, dtype=torch.int64).view(torch.float64)
+            for _ in range(3)]
+    for mask, nump in ((0b111, 3), (0b111, 4), (0b101, 2)):
+        want = O.manager_allreduce_(reps, mask_to_list(mask, 3), nump)
+        out = torch.empty(n, dtype=torch.float64, device=device)
+        ops.reduce_avg_(out, [r.to(device) for r in reps], mask, nump)
+        assert_bits_equal_up_to_nan_payload(out, want, f"mask {mask:#b} n {nump}")
+
+
 def test_reference_known_answers(device):
     # torchft/manager_test.py:520-543: 1.0 with 5 participants -> 0.2; healing -> 0.0
     t = torch.tensor([1.0], device=device)
@@ -282,7 +357,7 @@ def test_argument_errors(device):
     with pytest.raises(RuntimeError):
         ops.reduce_avg_(torch.zeros(8), [torch.zeros(8)])
     with pytest.raises(TypeError):
-        ops.reduce_avg_(x.double(), [x.double()])
+        ops.reduce_avg_(x.long(), [x.long()])
     with pytest.raises(ValueError):
         ops.reduce_avg_(torch.zeros(4, 4, device=device).t(), [x[:16]])
 

@@ -131,3 +131,98 @@ def test_sync_with_placed_buffers_matches_the_checker(device, kind, monkeypatch)
         torch.cuda.empty_cache()
     for x, y in zip(results["1"], results["0"]):
         assert_bits_equal(x, y)
+
+
+def _construct(model, device, kind="diloco"):
+    peer = [p.data + 1e-3 for p in model.parameters()]
+    index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    if kind == "diloco":
+        outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+        return DiLoCo(manager, model, inner, outer, sync_every=10 ** 9), manager, peer
+    return LocalSGD(manager, model, inner, sync_every=10 ** 9), manager, peer
+
+
+def test_a_second_construction_finds_the_groups_already_known(device):
+    """What the first search learnt about the device stays: the anchors are kept, and the blocks
+    of a dropped wrapper come back from torch's cache at addresses whose group is known.  The
+    second construction measures the model's own tensors and nothing else."""
+    import gc
+
+    H.forget_devices()
+    gc.collect()
+    torch.cuda.empty_cache()
+    torch.manual_seed(0)
+    model = Wide().to(device)
+    start = H.launch_count
+    ctx, manager, peer = _construct(model, device)
+    first = H.launch_count - start
+    state = H.device_state(device)
+    if ctx._placed_momentum is None:
+        pytest.skip("no bank-group structure found: is this an MI355X?")
+    assert state.searches == 1 and len(state.map.anchors) >= 2
+    anchors = [a.data_ptr() for a in state.map.anchors]
+    manager.shutdown(wait=False)
+    del ctx, manager
+    gc.collect()  # the wrapper's buffers go back to torch's cache, not to the driver
+    start = H.launch_count
+    ctx, manager, peer = _construct(model, device)
+    second = H.launch_count - start
+    assert state.searches == 2
+    assert [a.data_ptr() for a in state.map.anchors][:len(anchors)] == anchors
+    assert ctx._placed_momentum is not None
+    assert second < 0.1 * first, (first, second)
+    # and the buffers still lie outside the model's group
+    big, copy0 = model.a.data, ctx._backup_parameters["a"]
+    half = copy0.numel() // 2
+    for attempt in range(3):
+        same = H.probe_ms(copy0[:half], copy0[half:], 256 << 20, repeats=6)
+        ratio = H.probe_ms(big, copy0, 256 << 20, repeats=6) / same
+        if ratio < 0.92:
+            break
+    assert ratio < 0.92, ratio
+    manager.shutdown(wait=False)
+
+
+def test_two_replicas_constructing_at_once_take_turns(device):
+    """Two thread-replicas on one GPU build their wrappers at the same time: the searches run
+    one after the other under the device's lock, both get placed buffers that do not overlap,
+    and a sync of each equals the checker."""
+    import threading
+
+    torch.manual_seed(0)
+    models = [Wide().to(device) for _ in range(2)]
+    built = [None, None]
+    errors = []
+
+    def build(k):
+        try:
+            with torch.cuda.device(device):
+                built[k] = _construct(models[k], device, "local_sgd")
+        except Exception as e:  # surfaced below
+            errors.append(e)
+
+    threads = [threading.Thread(target=build, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    spans = []
+    for ctx, _, _ in built:
+        for b in ctx._backup_parameters.values():
+            spans.append((b.data_ptr(), b.data_ptr() + b.numel() * b.element_size()))
+    spans.sort()
+    assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(spans, spans[1:])), "buffers overlap"
+    for k, (ctx, manager, peer) in enumerate(built):
+        backup = [b.cpu() for b in ctx._backup_parameters.values()]
+        reps = [[p.data.cpu() for p in models[k].parameters()], [t.cpu() for t in peer]]
+        want = O.localsgd_perform_sync(reps, backup, [True, True], 2, True)
+        ctx.sync()
+        torch.cuda.synchronize()
+        for i, p in enumerate(models[k].parameters()):
+            assert_bits_equal(p.data, want["params"][i], f"replica {k} params[{i}]")
+        manager.shutdown(wait=False)

@@ -38,7 +38,7 @@ from torchft_amd import (
 from torchft_amd.checkpointing import _timed_acquire
 from torchft_amd.ddp import compute_bucket_assignment
 from torchft_amd.manager import QuorumClient
-from torchft_amd.process_group import _DummyWork
+from torchft_amd.process_group import ProcessGroupDummy, _DummyWork
 
 
 class SimpleModel(nn.Module):
@@ -890,6 +890,24 @@ def test_kernels_refuse_cpu_tensors():
         model(torch.rand(2, 3)).mean().backward()
         with pytest.raises(RuntimeError, match="no CPU path"):
             inner.step()
+
+
+def test_manager_allreduce_latches_what_the_kernels_cannot_take():
+    """torchft/manager.py:242-303 never raises; neither does this one.  A host tensor has no
+    kernel to run on (and there is no CPU arithmetic to fall back to): the error is latched,
+    the tensor comes back untouched and the step does not commit."""
+    manager = Manager(pg=ProcessGroupDummy(0, 1), load_state_dict=None, state_dict=None,
+                      min_replica_size=1)
+    manager.start_quorum()
+    t = torch.tensor([1.0, 2.0])
+    fut = manager.allreduce(t)
+    assert fut.wait() is t
+    assert isinstance(manager.errored(), RuntimeError) and "no CPU path" in str(manager.errored())
+    assert torch.equal(t, torch.tensor([1.0, 2.0]))
+    assert not manager.should_commit()
+    manager.start_quorum()
+    assert manager.errored() is None
+    manager.shutdown(wait=False)
 
 
 # ---------------------------------------------------------------------------

@@ -18,7 +18,7 @@ import torch  # noqa: F401  (must precede loading the library, see module docstr
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchft_amd.so"
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 MAX_REPLICAS = 8
 MIN_CHUNK_ELEMS = 8192
 MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
@@ -27,6 +27,7 @@ NOALLOC_MAX_TENSORS = 4096
 TFT_F32 = 0
 TFT_BF16 = 1
 TFT_F16 = 2
+TFT_F64 = 3  # replica average only
 
 
 class MtTable(Structure):

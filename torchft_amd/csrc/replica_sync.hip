@@ -52,6 +52,7 @@ int fail(int code, const char* fmt, ...) {
 // ---------------------------------------------------------------------------
 struct F32 {
   typedef float elem_t;
+  typedef float acc_t;  // the type the arithmetic runs in
   static constexpr int kVec = 4;
   __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
 #pragma unroll
@@ -78,6 +79,7 @@ __device__ inline uint32_t f32_to_bf16_bits(float f) {
 
 struct BF16 {
   typedef uint16_t elem_t;
+  typedef float acc_t;
   static constexpr int kVec = 8;
   __device__ static inline void widen(const u32x4& raw, float (&v)[kVec]) {
 #pragma unroll
@@ -107,6 +109,7 @@ struct BF16 {
 
 struct F16 {
   typedef uint16_t elem_t;
+  typedef float acc_t;
   static constexpr int kVec = 8;
   __device__ static inline float widen1(uint16_t x) { return __half2float(__ushort_as_half(x)); }
   __device__ static inline uint16_t narrow1(float x) {
@@ -132,6 +135,37 @@ struct F16 {
     return raw;
   }
 };
+
+// fp64: two elements per 128-bit access, arithmetic in fp64 (only the replica
+// average is instantiated for it: Manager.allreduce is dtype-generic in the
+// reference, torchft/manager.py:267-287)
+struct F64 {
+  typedef double elem_t;
+  typedef double acc_t;
+  static constexpr int kVec = 2;
+  __device__ static inline void widen(const u32x4& raw, double (&v)[kVec]) {
+    v[0] = __hiloint2double((int)raw[1], (int)raw[0]);
+    v[1] = __hiloint2double((int)raw[3], (int)raw[2]);
+  }
+  __device__ static inline u32x4 narrow(const double (&v)[kVec]) {
+    u32x4 raw;
+    raw[0] = (uint32_t)__double2loint(v[0]);
+    raw[1] = (uint32_t)__double2hiint(v[0]);
+    raw[2] = (uint32_t)__double2loint(v[1]);
+    raw[3] = (uint32_t)__double2hiint(v[1]);
+    return raw;
+  }
+  __device__ static inline double widen1(double x) { return x; }
+  __device__ static inline double narrow1(double x) { return x; }
+};
+
+// round-to-nearest arithmetic the compiler may not contract or re-associate, by type
+__device__ inline float add_rn(float a, float b) { return __fadd_rn(a, b); }
+__device__ inline double add_rn(double a, double b) { return __dadd_rn(a, b); }
+__device__ inline float mul_rn(float a, float b) { return __fmul_rn(a, b); }
+__device__ inline double mul_rn(double a, double b) { return __dmul_rn(a, b); }
+__device__ inline float div_rn(float a, float b) { return __fdiv_rn(a, b); }
+__device__ inline double div_rn(double a, double b) { return __ddiv_rn(a, b); }
 
 template <bool NT>
 __device__ inline u32x4 load16(const void* p) {
@@ -296,12 +330,12 @@ __device__ inline void stream_block(char* const (&ptr)[Op::NCOL], const Op& op, 
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    float lanes[NCOL][V];
+    typename E::acc_t lanes[NCOL][V];
 #pragma unroll
     for (int c = 0; c < NCOL; ++c) E::widen(raw[c][u], lanes[c]);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      float v[NCOL];
+      typename E::acc_t v[NCOL];
 #pragma unroll
       for (int c = 0; c < NCOL; ++c) v[c] = lanes[c][i];
       if constexpr (FAST)
@@ -332,10 +366,10 @@ __device__ inline void scalar_range(char* const (&ptr)[Op::NCOL], const Op& op, 
   constexpr int NCOL = Op::NCOL;
   typedef typename E::elem_t T;
   for (uint32_t i = begin + threadIdx.x; i < end; i += kThreads) {
-    float v[NCOL];
+    typename E::acc_t v[NCOL];
 #pragma unroll
     for (int c = 0; c < NCOL; ++c)
-      v[c] = ((rmask >> c) & 1u) ? E::widen1(reinterpret_cast<const T*>(ptr[c])[i]) : 0.0f;
+      v[c] = ((rmask >> c) & 1u) ? E::widen1(reinterpret_cast<const T*>(ptr[c])[i]) : 0;
     op.apply(v);
 #pragma unroll
     for (int c = 0; c < NCOL; ++c)
@@ -390,19 +424,26 @@ __global__ __launch_bounds__(kThreads) void mt_stream_kernel(typename Loc::args_
 // the IEEE division bit for bit: inv is that reciprocal, or 0 when n is no power of two.
 struct Divisor {
   float n, inv;
+  uint32_t count;  // the integer itself (fp64 arithmetic converts it exactly)
+  __device__ inline float as(float) const { return n; }
+  __device__ inline double as(double) const { return (double)count; }
+  // the reciprocal is a power of two: exact in either type
+  __device__ inline float inverse(float) const { return inv; }
+  __device__ inline double inverse(double) const { return (double)inv; }
 };
 
 Divisor make_divisor(uint32_t num_participants) {
   const bool pow2 = num_participants && !(num_participants & (num_participants - 1u));
-  return Divisor{(float)num_participants, pow2 ? 1.0f / (float)num_participants : 0.0f};
+  return Divisor{(float)num_participants, pow2 ? 1.0f / (float)num_participants : 0.0f,
+                 num_participants};
 }
 
-template <int NREP>
-__device__ inline float replica_sum(const float* x, uint32_t mask) {
+template <int NREP, class T>
+__device__ inline T replica_sum(const T* x, uint32_t mask) {
   // sequential in replica order; a non-participant contributes +0
-  float s = (mask & 1u) ? x[0] : 0.0f;
+  T s = (mask & 1u) ? x[0] : T(0);
 #pragma unroll
-  for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, ((mask >> r) & 1u) ? x[r] : 0.0f);
+  for (int r = 1; r < NREP; ++r) s = add_rn(s, ((mask >> r) & 1u) ? x[r] : T(0));
   return s;
 }
 
@@ -415,20 +456,22 @@ struct ReduceAvgOp {
   Divisor d;      // num_participants
   __device__ inline uint32_t rmask() const { return mask << NOUT; }
   __device__ inline uint32_t wmask() const { return (1u << NOUT) - 1u; }
-  __device__ inline void apply(float (&v)[NCOL]) const {
-    float s = 0.0f;
-    if constexpr (NREP > 0) s = replica_sum<NREP>(&v[NOUT], mask);
-    s = __fdiv_rn(s, d.n);
+  template <class T>
+  __device__ inline void apply(T (&v)[NCOL]) const {
+    T s = T(0);
+    if constexpr (NREP > 0) s = replica_sum<NREP, T>(&v[NOUT], mask);
+    s = div_rn(s, d.as(T()));
 #pragma unroll
     for (int o = 0; o < NOUT; ++o) v[o] = s;
   }
   // everybody participates and the divisor is a power of two
   __device__ inline bool fast() const { return mask == (1u << NREP) - 1u && d.inv != 0.0f; }
-  __device__ inline void apply_fast(float (&v)[NCOL]) const {
-    float s = v[NOUT];
+  template <class T>
+  __device__ inline void apply_fast(T (&v)[NCOL]) const {
+    T s = v[NOUT];
 #pragma unroll
-    for (int r = 1; r < NREP; ++r) s = __fadd_rn(s, v[NOUT + r]);
-    s = __fmul_rn(s, d.inv);
+    for (int r = 1; r < NREP; ++r) s = add_rn(s, v[NOUT + r]);
+    s = mul_rn(s, d.inverse(T()));
 #pragma unroll
     for (int o = 0; o < NOUT; ++o) v[o] = s;
   }
@@ -771,7 +814,11 @@ int check_reduce(const char* what, uint32_t n_replicas, uint32_t mask, uint32_t 
   return TFT_OK;
 }
 
-int check_dtype(const char* what, int dtype) {
+// fp64 exists for the replica average only (allow_f64)
+int check_dtype(const char* what, int dtype, bool allow_f64 = false) {
+  if (dtype == TFT_F64 && allow_f64) return TFT_OK;
+  if (dtype == TFT_F64)
+    return fail(TFT_ERR_UNSUPPORTED, "%s: fp64 is supported by the replica average only", what);
   if (dtype != TFT_F32 && dtype != TFT_BF16 && dtype != TFT_F16)
     return fail(TFT_ERR_UNSUPPORTED, "%s: dtype %d", what, dtype);
   return TFT_OK;
@@ -855,6 +902,13 @@ int launch_flat(const char* what, const FlatArgs& args, const Op& op, const Shap
     else TFT_DISPATCH_U(rc, LAUNCHER, F16, OP, what, ARGS, op, shape, stream);                           \
   } while (0)
 
+// The replica average also exists for fp64.
+#define TFT_DISPATCH_DTYPE_F64(rc, LAUNCHER, OP, dtype, what, ARGS, op, shape, stream)           \
+  do {                                                                                          \
+    if ((dtype) == TFT_F64) TFT_DISPATCH_U(rc, LAUNCHER, F64, OP, what, ARGS, op, shape, stream); \
+    else TFT_DISPATCH_DTYPE(rc, LAUNCHER, OP, dtype, what, ARGS, op, shape, stream);            \
+  } while (0)
+
 // Expands `CALL(N)` for the run-time replica count.
 #define TFT_FOR_NREP(n, CALL) \
   switch (n) {                \
@@ -889,7 +943,7 @@ int check_sgd(const char* what, const tft_sgd_params* s) {
   return TFT_OK;
 }
 
-uint64_t esize_of(int dtype) { return dtype == TFT_F32 ? 4 : 2; }
+uint64_t esize_of(int dtype) { return dtype == TFT_F64 ? 8 : dtype == TFT_F32 ? 4 : 2; }
 
 // elements a table covers, rounded up to whole chunks (the host does not read the
 // device-resident sizes); only used to choose the launch shape
@@ -999,7 +1053,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
                    int dtype, void* stream) {
   static const char* what = "tft_reduce_avg";
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (int rc = check_dtype(what, dtype)) return rc;
+  if (int rc = check_dtype(what, dtype, true)) return rc;
   if (numel == 0) return TFT_OK;
   if (!out) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: out is NULL", what);
   if (n_replicas && !replicas) return fail(TFT_ERR_INVALID_ARGUMENT, "%s: replicas is NULL", what);
@@ -1020,7 +1074,7 @@ int tft_reduce_avg(void* out, const void* const* replicas, uint32_t n_replicas,
   do {                                                                          \
     typedef ReduceAvgOp<1, N> Op;                                               \
     const Op op{participate_mask, make_divisor(num_participants)};              \
-    TFT_DISPATCH_DTYPE(rc, launch_flat, Op, dtype, what, a, op, shape, s);      \
+    TFT_DISPATCH_DTYPE_F64(rc, launch_flat, Op, dtype, what, a, op, shape, s);  \
   } while (0)
   TFT_FOR_NREP(n_replicas, TFT_CALL)
 #undef TFT_CALL
@@ -1034,7 +1088,7 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
   if (n_outs != 1 && n_outs != 2)
     return fail(TFT_ERR_INVALID_ARGUMENT, "%s: n_outs must be 1 or 2, got %u", what, n_outs);
   if (int rc = check_reduce(what, n_replicas, participate_mask, num_participants)) return rc;
-  if (int rc = check_dtype(what, dtype)) return rc;
+  if (int rc = check_dtype(what, dtype, true)) return rc;
   if (int rc = check_table(what, table, n_outs + n_replicas)) return rc < 0 ? rc : TFT_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Shape shape = pick_shape(
@@ -1044,7 +1098,7 @@ int tft_mt_reduce_avg(const tft_mt_table* table, uint32_t n_outs, uint32_t n_rep
   do {                                                                                \
     typedef ReduceAvgOp<O, N> Op;                                                     \
     const Op op{participate_mask, make_divisor(num_participants)};                    \
-    TFT_DISPATCH_DTYPE(rc, launch_table, Op, dtype, what, table, op, shape, s);       \
+    TFT_DISPATCH_DTYPE_F64(rc, launch_table, Op, dtype, what, table, op, shape, s);   \
   } while (0)
 #define TFT_CALL_O1(N) TFT_CALL2(1, N)
 #define TFT_CALL_O2(N) TFT_CALL2(2, N)

@@ -45,7 +45,8 @@ from .multi_tensor import TensorTable
 logger: logging.Logger = logging.getLogger(__name__)
 
 
-_KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+_KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)   # every kernel
+_AVERAGE_DTYPES = _KERNEL_DTYPES + (torch.float64,)                # the replica average and the copies
 
 _DATA_PTR = torch.Tensor.data_ptr
 _NUMEL = torch.Tensor.numel
@@ -156,6 +157,8 @@ class LocalSGD:
     fault tolerant: if anything fails between two syncs the parameters roll back to
     the backup taken at the last successful sync (torchft/local_sgd.py:26-175)."""
 
+    _DTYPES = _AVERAGE_DTYPES
+
     def __init__(
         self,
         manager: Manager,
@@ -226,11 +229,11 @@ class LocalSGD:
             _native.lib()  # GPU parameters need the kernels: fail now, loudly, if they are missing
             # a dtype the kernels do not have is a configuration error: say so here, once,
             # instead of latching it as a failed all-reduce on every sync
-            bad = sorted({str(p.dtype) for _, p in named if p.is_cuda and p.dtype not in _KERNEL_DTYPES})
+            bad = sorted({str(p.dtype) for _, p in named if p.is_cuda and p.dtype not in self._DTYPES})
             if bad:
                 raise TypeError(
-                    f"{type(self).__name__}: GPU parameters of {', '.join(bad)}; the replica-sync "
-                    "kernels take float32, bfloat16 and float16"
+                    f"{type(self).__name__}: GPU parameters of {', '.join(bad)}; its kernels take "
+                    + ", ".join(str(d).replace("torch.", "") for d in self._DTYPES)
                 )
         # the first sync needs a valid backup
         self._save_parameters()
@@ -516,6 +519,8 @@ class DiLoCo(LocalSGD):
     """DiLoCo (https://arxiv.org/pdf/2311.08105): the replicas average their
     pseudo-gradients ``params - backup`` and an outer optimizer applies the average
     to the parameters restored from the backup (torchft/local_sgd.py:177-239)."""
+
+    _DTYPES = _KERNEL_DTYPES  # the outer step's arithmetic is fp32
 
     def __init__(
         self,

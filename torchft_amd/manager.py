@@ -451,14 +451,16 @@ class Manager(Generic[T]):
 
         Never raises: a failure is latched (``errored()``), the future still
         completes with the (possibly corrupt) tensor and every later call is a no-op
-        until the next ``start_quorum`` (torchft/manager.py:242-303).  The one exception is
-        a tensor the kernels cannot take at all (CPU, non-contiguous, unsupported dtype):
-        that is a configuration error and raises, instead of blocking every commit."""
-        ops.check_tensor(tensor, "Manager.allreduce")
+        until the next ``start_quorum`` (torchft/manager.py:242-303).  That includes a
+        tensor the kernels cannot take (not on a GPU, not contiguous, an integer dtype):
+        it is reported and latched like any other failed all-reduce, so the step is
+        discarded instead of the training loop being torn down.  There is no CPU
+        arithmetic behind this method."""
         if self.errored():
             return _done_future(tensor)
         self.wait_quorum()
         try:
+            ops.check_tensor(tensor, "Manager.allreduce")
             if hasattr(self._pg, "allreduce_avg"):
                 work = self._pg.allreduce_avg(
                     [tensor], self.is_participating(), self.num_participants()

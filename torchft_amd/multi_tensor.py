@@ -23,6 +23,7 @@ _DTYPE_CODES = {
     torch.float32: _native.TFT_F32,
     torch.bfloat16: _native.TFT_BF16,
     torch.float16: _native.TFT_F16,
+    torch.float64: _native.TFT_F64,  # the replica average only
 }
 
 
@@ -36,7 +37,8 @@ def dtype_code(dtype: torch.dtype) -> int:
         return _DTYPE_CODES[dtype]
     except KeyError:
         raise TypeError(
-            f"torchft_amd kernels support float32, bfloat16 and float16, got {dtype}"
+            f"torchft_amd kernels support float32, bfloat16, float16 and (replica average only) "
+            f"float64, got {dtype}"
         ) from None
 
 

@@ -46,8 +46,8 @@ class OuterSGD:
 
 
 def check_tensor(t: torch.Tensor, what: str) -> None:
-    """Raises for a tensor no kernel can take (not on a GPU, not contiguous, or of a dtype
-    other than fp32 / bf16 / fp16): a configuration error, never a transient failure."""
+    """Raises for a tensor the replica average cannot take: not on a GPU, not contiguous, or
+    of a dtype other than fp32 / bf16 / fp16 / fp64."""
     require_device_tensor(t, what)
     dtype_code(t.dtype)
 
