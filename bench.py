@@ -51,6 +51,7 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=WORKLOADS, default=WORKLOADS[0])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--recv-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-api", action="store_true",
                     help="headline workload: leave out the sub-record measured through DiLoCo.sync()")
     ap.add_argument("--cpu-layers", type=int, default=8,
@@ -1095,7 +1096,7 @@ def bench_checkpoint(args) -> Dict[str, object]:
             "sample": f"training state of 1 of 32 decoder layers on the GPU ({small_bytes} bytes), one "
                       f"torch.save into memory + torch.load (the reference's send / receive seats), "
                       f"{dt:.2f} s; includes its per-storage device-to-host copies"}
-    out["http_recovery"] = http_recovery(dev)
+    out["http_recovery"] = http_recovery(dev, getattr(args, "child", None))
     out["pcie"] = {"d2h_GBs": total / d2h_s / 1e9, "h2d_GBs": total / h2d_s / 1e9,
                    "d2h_s": d2h_s, "h2d_s": h2d_s, "bytes": total,
                    "note": "staging buffer through two 1 GiB pinned bounce buffers; PCIe-bound, "
@@ -1114,12 +1115,112 @@ class _Discard:
         return len(view)
 
 
-def http_recovery(dev: torch.device) -> Dict[str, object]:
+def recv_child() -> int:
+    """The receiving replica of ``http_recovery`` as a process of its own (started before the
+    parent touches the GPU): reads one JSON command per line from stdin, answers one JSON line.
+    ``fetch``: recover a state from a CheckpointServer address onto this process's GPU context;
+    ``sink``: receive plain bytes over k loopback TCP connections into pinned buffers (what the
+    kernel's loopback path allows a Python receiver, with no GPU and no HTTP involved)."""
+    import socket
+    import threading
+    from datetime import timedelta
+
+    from torchft_amd import CheckpointServer, state_pack
+
+    torch.cuda.set_device(0)
+    torch.zeros(1, device="cuda")  # context up before the first timed command
+    for line in sys.stdin:
+        cmd = json.loads(line)
+        if cmd["op"] == "quit":
+            break
+        if cmd["op"] == "fetch":
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            got = CheckpointServer.load_from_address(cmd["address"], timedelta(seconds=120),
+                                                     streams=cmd["streams"])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            t = got["user"]["model"][cmd["name"]]
+            checksum = int(t.view(torch.int16).sum(dtype=torch.int64))
+            del got, t
+            print(json.dumps({"seconds": dt, "checksum": checksum}), flush=True)
+        elif cmd["op"] == "sink":
+            k, per_conn, chunk = cmd["connections"], cmd["bytes_per_connection"], 64 << 20
+            bufs = [state_pack.PINNED.acquire(chunk) for _ in range(k)]
+
+            def drain(j: int) -> None:
+                view = memoryview(bufs[j].numpy())
+                with socket.create_connection(("127.0.0.1", cmd["port"])) as c:
+                    left = per_conn
+                    while left:
+                        n = c.recv_into(view[:min(chunk, left)])
+                        if not n:
+                            raise EOFError("sender closed early")
+                        left -= n
+
+            threads = [threading.Thread(target=drain, args=(j,)) for j in range(k)]
+            t0 = time.perf_counter()
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+            dt = time.perf_counter() - t0
+            for b in bufs:
+                state_pack.PINNED.release(b)
+            print(json.dumps({"seconds": dt}), flush=True)
+    return 0
+
+
+def loopback_bound(child, connections: int, bytes_per_connection: int) -> float:
+    """GB/s of plain loopback TCP from pinned buffers of this process into pinned buffers of
+    the child over ``connections`` sockets: the ceiling of any recovery between two processes
+    of one host, whatever is done on the GPU side."""
+    import socket
+    import threading
+
+    from torchft_amd import state_pack
+
+    chunk = 64 << 20
+    srv = socket.socket(socket.AF_INET, socket.SOCK_STREAM)
+    srv.setsockopt(socket.SOL_SOCKET, socket.SO_REUSEADDR, 1)
+    srv.bind(("127.0.0.1", 0))
+    srv.listen(connections)
+    bufs = [state_pack.PINNED.acquire(chunk) for _ in range(connections)]
+
+    def feed(conn, j: int) -> None:
+        view = memoryview(bufs[j].numpy())
+        with conn:
+            left = bytes_per_connection
+            while left:
+                n = min(chunk, left)
+                conn.sendall(view[:n])
+                left -= n
+
+    child.stdin.write(json.dumps({"op": "sink", "port": srv.getsockname()[1], "connections": connections,
+                                  "bytes_per_connection": bytes_per_connection}) + "\n")
+    child.stdin.flush()
+    threads = []
+    for j in range(connections):
+        conn, _ = srv.accept()
+        threads.append(threading.Thread(target=feed, args=(conn, j)))
+        threads[-1].start()
+    for t in threads:
+        t.join()
+    answer = json.loads(child.stdout.readline())
+    srv.close()
+    for b in bufs:
+        state_pack.PINNED.release(b)
+    return connections * bytes_per_connection / answer["seconds"] / 1e9
+
+
+def http_recovery(dev: torch.device, child=None) -> Dict[str, object]:
     """Live recovery end to end on a bounded slice: CheckpointServer.send_checkpoint on one
-    side, recv_checkpoint on the other (same process, loopback HTTP): chunks gathered on the
-    device into a ring, pinned D2H, socket, pinned H2D, views on the receiving GPU; with 1, 2,
-    4 and 8 parallel connections.  Also the serving pipeline alone (same chunks into a sink
-    instead of a socket), which is what PCIe allows."""
+    side, recv_checkpoint on the other over loopback HTTP: chunks gathered on the device into
+    a ring, pinned D2H, socket, pinned H2D, views on the receiving GPU; with 1, 2, 4 and 8
+    parallel connections.  The receiver runs once inside this process (sender and receiver
+    share one interpreter lock) and once as a process of its own (``child``), next to what
+    plain loopback TCP between the two processes carries.  Also the serving pipeline alone
+    (same chunks into a sink instead of a socket), which is what PCIe allows."""
     from datetime import timedelta
 
     from torchft_amd import CheckpointServer, state_pack, workloads
@@ -1133,8 +1234,9 @@ def http_recovery(dev: torch.device) -> Dict[str, object]:
     t0 = time.perf_counter()
     state_pack.stream_packed(plan, sink)
     pipeline_s = time.perf_counter() - t0
-    rates = {}
+    rates, child_rates, bound = {}, {}, {}
     name = next(iter(state["user"]["model"]))
+    want_sum = int(state["user"]["model"][name].view(torch.int16).sum(dtype=torch.int64))
     for streams in (1, 2, 4, 8):
         server = CheckpointServer(timeout=timedelta(seconds=120), fetch_streams=streams)
         try:
@@ -1148,19 +1250,38 @@ def http_recovery(dev: torch.device) -> Dict[str, object]:
                 raise RuntimeError("recovered state differs")
             rates[str(streams)] = nbytes / dt / 1e9
             del got
+            if child is not None:
+                for attempt in range(2):  # the first fetch of the child pins its buffers
+                    child.stdin.write(json.dumps({"op": "fetch", "address": f"{server.metadata()}1",
+                                                  "streams": streams, "name": name}) + "\n")
+                    child.stdin.flush()
+                    answer = json.loads(child.stdout.readline())
+                    if answer["checksum"] != want_sum:
+                        raise RuntimeError("state recovered by the child process differs")
+                child_rates[str(streams)] = nbytes / answer["seconds"] / 1e9
         finally:
             server.shutdown()
-    return {"GBs_by_connections": rates, "serving_pipeline_to_pinned_host_GBs": nbytes / pipeline_s / 1e9,
-            "bytes": nbytes,
-            "note": "training state of 4 decoder layers served and fetched over loopback HTTP in one "
-                    "process; one connection is bound by Python socket I/O (a single TCP stream), "
-                    "which is why a recovery fetches byte ranges over several; the serving pipeline "
-                    "alone (device ring -> pinned host, no socket) shows the PCIe bound; the "
-                    "reference's torch.save / torch.load seats are timed in cpu_baseline"}
+    if child is not None:
+        for k in (1, 4, 8):
+            loopback_bound(child, k, 256 << 20)  # warm-up: pins, connects
+            bound[str(k)] = loopback_bound(child, k, (8 << 30) // k)
+    out = {"GBs_by_connections": rates, "serving_pipeline_to_pinned_host_GBs": nbytes / pipeline_s / 1e9,
+           "bytes": nbytes,
+           "note": "training state of 4 decoder layers served and fetched over loopback HTTP; one "
+                   "connection is bound by one TCP stream's two copies through the kernel, "
+                   "which is why a recovery fetches byte ranges over several; the serving pipeline "
+                   "alone (device ring -> pinned host, no socket) shows the PCIe bound; the "
+                   "reference's torch.save / torch.load seats are timed in cpu_baseline"}
+    if child is not None:
+        out["GBs_by_connections_receiver_in_its_own_process"] = child_rates
+        out["plain_loopback_tcp_between_the_two_processes_GBs"] = bound
+    return out
 
 
 def main() -> int:
     args = parse_args()
+    if args.recv_child:
+        return recv_child()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (asked for --gpus {args.gpus}); "
               "the N-replica reduction is simulated over N buffers resident on that GPU",
@@ -1169,6 +1290,13 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
+    if args.workload == "checkpoint_llama3_8b":
+        # the receiving replica of the recovery measurement: a process of its own, started
+        # before this one initialises the GPU
+        import subprocess
+
+        args.child = subprocess.Popen([sys.executable, "-u", os.path.abspath(__file__), "--recv-child"],
+                                      stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     if "no_placement" in args.layout.split(","):
         os.environ["TORCHFT_AMD_HBM_PLACEMENT"] = "0"
     if args.settle_seconds > 0:
@@ -1218,6 +1346,14 @@ def main() -> int:
         out = bench_host_backup(args)
     else:
         out = bench_localsgd(args)
+    child = getattr(args, "child", None)
+    if child is not None:
+        try:
+            child.stdin.write(json.dumps({"op": "quit"}) + "\n")
+            child.stdin.flush()
+            child.wait(timeout=30)
+        except Exception:
+            child.kill()
     print(json.dumps(out), flush=True)
     return 0
 

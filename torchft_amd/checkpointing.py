@@ -102,9 +102,10 @@ class CheckpointServer(CheckpointTransport[T]):
     """HTTP server that serves the current state dict, packed on the device.
 
     The gather kernels and the device-to-host copies of a request run on streams
-    of their own, ordered after whatever the training stream had enqueued when
-    ``send_checkpoint`` was called, so serving does not serialise with the
-    training thread's later work.  Requests for parts of one payload are served
+    of their own (pooled, with their device rings, between requests), ordered after
+    whatever the training stream had enqueued when ``send_checkpoint`` was called
+    and after nothing else, so serving does not serialise with the training
+    thread's later work.  Requests for parts of one payload are served
     concurrently; ``disallow_checkpoint`` closes the gate and waits until the
     requests in flight have stopped reading the state.
     """
@@ -235,6 +236,8 @@ class CheckpointServer(CheckpointTransport[T]):
                 try:
                     with torch.cuda.device(device):
                         lo, hi = state_pack.split_range(total, part, streams)
+                        if lo >= hi:
+                            return  # a small payload does not fill every range: nothing to ask for
                         with urllib.request.urlopen(f"{address}?part={part}&of={streams}", timeout=seconds) as g:
                             if state_pack.read_header(g) != header:
                                 raise RuntimeError("the served state changed between two parts of one fetch")

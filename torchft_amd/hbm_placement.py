@@ -144,7 +144,7 @@ class _Block:
     storage: torch.Tensor  # uint8, BLOCK_BYTES (or larger for a tensor that needs it)
     group: int
     used: int = 0
-    floor: int = 0         # bytes at the start that are never handed out (an anchor lives there)
+    floor: int = 0         # bytes at the start that are never handed out
 
     def free(self) -> int:
         return self.storage.numel() - max(self.used, self.floor)
@@ -211,8 +211,8 @@ class DeviceState:
         self.device = device
         self.lock = threading.RLock()
         self.map = GroupMap(device)
-        # blocks whose first PROBE_BYTES are an anchor: never returned; the rest of each is
-        # handed out once (it is not reclaimed when the tensors carved from it die)
+        # blocks an end of which had to serve as an anchor itself (rare: see _found_group):
+        # never handed out, never returned
         self.anchor_blocks: List[_Block] = []
         # address of a block classified earlier -> (bytes, group); valid while torch's
         # allocator has not given memory back to the driver since (``epoch``)
@@ -220,6 +220,7 @@ class DeviceState:
         self.epoch: Optional[int] = None
         self.structured = True   # False once the timings have shown no group structure
         self.searches = 0
+        self.last_search: Dict[str, float] = {}  # figures of the most recent search (also logged)
 
 
 _STATES: Dict[Tuple[str, int], DeviceState] = {}
@@ -270,8 +271,7 @@ class GroupedPool:
         self.device = device
         self.state = state if state is not None else DeviceState(device)
         self.map = self.state.map
-        # the unreserved rest of the anchors' blocks is the first memory of known group
-        self.blocks: List[_Block] = list(self.state.anchor_blocks)
+        self.blocks: List[_Block] = []
         self._straddling: List[torch.Tensor] = []  # blocks across a group boundary: held, unused
         # where blocks come from and go back to (replaceable: the search logic is host code
         # and is tested without a GPU)
@@ -283,7 +283,8 @@ class GroupedPool:
         self.keep_free = 6 << 30  # device memory the search never touches
         self.limit: Optional[int] = None  # bytes this search may hold; None: search_limit_bytes
         self.held = 0             # bytes taken from the device by this search
-        self.cache_hits = 0
+        self.cache_hits = 0       # blocks whose group was known by their address
+        self.blocks_probed = 0    # blocks whose group had to be measured
         if self.state.epoch is not None and self.state.epoch != self._epoch():
             self.state.known.clear()  # memory went back to the driver: addresses mean nothing now
 
@@ -293,41 +294,48 @@ class GroupedPool:
 
     # -- discovery ---------------------------------------------------------------
     def _classify_block(self, block: _Block) -> Optional[int]:
-        """Group of a fresh block (a new anchor is made of it if its group is new); None if
-        the block straddles two groups."""
+        """Group of a fresh block (a new anchor is set up next to it if its group is new); None
+        if the block straddles two groups."""
         m = self.map
         storage = block.storage
-        if not m.anchors:
-            m.anchors.append(storage[:PROBE_BYTES])
-            self._keep_as_anchor(block)
-            return 0
         n = storage.numel()
         ends = []
         for piece in (storage[:PROBE_BYTES], storage[n - PROBE_BYTES:]):
             g = m.group_of(piece)
             if g is None:
-                if len(m.anchors) >= N_GROUPS or not self._clearly_new(storage):
+                if len(m.anchors) >= N_GROUPS or not self._clearly_new(piece):
                     return None  # matches no group clearly: leave it alone
-                m.anchors.append(piece)
-                self._keep_as_anchor(block, at_end=piece.data_ptr() != storage.data_ptr())
-                g = len(m.anchors) - 1
+                g = self._found_group(piece, block)
             ends.append(g)
         return ends[0] if ends[0] == ends[1] else None
 
-    def _keep_as_anchor(self, block: _Block, at_end: bool = False) -> None:
-        if at_end:
-            # the anchor is the block's tail (a block across a boundary founded the group):
-            # nothing of it is handed out
+    def _found_group(self, piece: torch.Tensor, block: _Block) -> int:
+        """``piece`` (an end of ``block``) lies in a group no anchor is known for.  The anchor
+        becomes a small allocation of its own, taken right now: the driver hands memory out
+        in address order, so it lies right behind the block - which is checked.  The block
+        itself then stays an ordinary block.  Only if that check fails is the piece itself
+        kept as the anchor (and its block never handed out or returned)."""
+        m = self.map
+        anchor: Optional[torch.Tensor] = None
+        try:
+            candidate = self._allocate(PROBE_BYTES)
+            n = min(piece.numel(), candidate.numel()) // 16 * 16
+            if probe_ms(piece, candidate, n, repeats=5) / m._same_ms(n) > SAME_GROUP_RATIO + AMBIGUOUS_BAND:
+                anchor = candidate
+        except Exception as e:  # no room for it: fall back to the piece
+            logger.info("hbm placement: no separate anchor (%s)", e)
+        if anchor is None:
+            anchor = piece
             block.floor = block.storage.numel()
-        else:
-            block.floor = min(PROBE_BYTES, block.storage.numel())
-        self.state.anchor_blocks.append(block)
+            self.state.anchor_blocks.append(block)
+        m.anchors.append(anchor)
+        return len(m.anchors) - 1
 
     def _clearly_new(self, storage: torch.Tensor) -> bool:
-        """A second, longer measurement before a block founds a new group: an anchor that in
+        """A second, longer measurement before a piece founds a new group: an anchor that in
         truth lies in a known group would make every later block of that group unclassifiable."""
         m = self.map
-        n = min(storage.numel(), 2 * PROBE_BYTES) // 16 * 16
+        n = min(storage.numel(), PROBE_BYTES) // 16 * 16
         same = m._same_ms(n)
         return all(probe_ms(storage, anchor, n, repeats=9) / same < SAME_GROUP_RATIO - AMBIGUOUS_BAND
                    for anchor in m.anchors)
@@ -356,6 +364,10 @@ class GroupedPool:
                 logger.info("hbm placement: the search stops at its allowance of %.1f GiB",
                             self.limit / (1 << 30))
                 return False
+            if not self.map.anchors:
+                # the first reference buffer: an allocation of its own (like every anchor), kept
+                # until the process ends; the blocks that follow are compared with it
+                self.map.anchors.append(self._allocate(PROBE_BYTES))
             storage = self._allocate(block_bytes)
             self.held += block_bytes
             block = _Block(storage, -1)
@@ -365,6 +377,7 @@ class GroupedPool:
                 self.cache_hits += 1
             else:
                 g = self._classify_block(block)
+                self.blocks_probed += 1
             if g is None:
                 self._straddling.append(storage)
             else:
@@ -398,12 +411,12 @@ class GroupedPool:
             b.used = 0
 
     def release_unused(self) -> None:
-        """Gives every block nothing was taken from back to the device (anchors stay)."""
-        anchors = self.state.anchor_blocks
+        """Gives every block nothing was taken from back to the device (the anchors, which are
+        allocations of their own, stay)."""
         for b in self.blocks:
-            if b.used == 0 and b not in anchors:
+            if b.used == 0:
                 self.state.known.pop(b.storage.data_ptr(), None)
-        self.blocks = [b for b in self.blocks if b.used > 0 or b in anchors]
+        self.blocks = [b for b in self.blocks if b.used > 0]
         self._straddling = []
         self.held = 0
         self._release()
@@ -530,14 +543,36 @@ def _allocate_apart(
     # a tensor in none of the known groups lies in the one not reached yet: every known group
     # is "another group" for it; the first is as good as any
     wanted = [((0 if g is None else g + 1) % n_known) for g in groups]
+    order = sorted(range(len(like)), key=lambda i: -sizes[i])  # large tensors first: they pack better
     need: Dict[int, int] = {}
     for size, w in zip(sizes, wanted):
         need[w] = need.get(w, 0) + n_copies * (-(-size // ALIGN) * ALIGN)
-    # head room for blocks that cannot be filled to the last byte
-    need = {g: n + block for g, n in need.items() if n > 0}
-    pool.grow_until(lambda pl: all(pl.free_bytes(g) >= n for g, n in need.items()), block_bytes=block)
+
+    def everything_fits(pl: GroupedPool) -> bool:
+        """Enough bytes in every wanted group, and (only then worth the walk) a dry run of the
+        hand-out itself: blocks cannot be filled to the last byte, and how many more it takes
+        depends on the sizes."""
+        if any(pl.free_bytes(g) < n for g, n in need.items()):
+            return False
+        cursors = {id(b): max(b.used, b.floor) for b in pl.blocks}
+        by_group: Dict[int, List[_Block]] = {}
+        for b in pl.blocks:
+            by_group.setdefault(b.group, []).append(b)
+        for i in order:
+            if not sizes[i]:
+                continue
+            for _ in range(n_copies):
+                for b in by_group.get(wanted[i], ()):
+                    start = -(-cursors[id(b)] // ALIGN) * ALIGN
+                    if start + sizes[i] <= b.storage.numel():
+                        cursors[id(b)] = start + sizes[i]
+                        break
+                else:
+                    return False
+        return True
+
+    pool.grow_until(everything_fits, block_bytes=block)
     n_groups = len(pool.map.anchors)
-    order = sorted(range(len(like)), key=lambda i: -sizes[i])  # large tensors first: they pack better
     placed: Dict[Tuple[int, int], Optional[torch.Tensor]] = {}
     misplaced = 0
     for i in order:
@@ -561,11 +596,18 @@ def _allocate_apart(
             raw = pool._allocate(max(sizes[i], 1))[: sizes[i]]
         placed[(i, k)] = raw.view(like[i].dtype).view(like[i].shape)
     copies = [[placed[(i, k)] for i in range(len(like))] for k in range(n_copies)]
+    pool.state.last_search = {
+        "seconds": time.perf_counter() - t0, "probe_launches": launch_count - launches0,
+        "blocks_probed": pool.blocks_probed, "blocks_known_by_address": pool.cache_hits,
+        "held_bytes": held, "misplaced": misplaced,
+    }
     logger.info(
         "hbm placement: %d tensors x %d copies over %d bank groups (%d not in their preferred group); "
-        "search %d on %s: %.2f s, %d probe launches, %d blocks known by address, %.1f GiB held at most",
+        "search %d on %s: %.2f s, %d probe launches, %d blocks measured, %d known by address, "
+        "%.1f GiB held at most",
         len(like), n_copies, n_groups, misplaced, pool.state.searches, device,
-        time.perf_counter() - t0, launch_count - launches0, pool.cache_hits, held / (1 << 30),
+        time.perf_counter() - t0, launch_count - launches0, pool.blocks_probed, pool.cache_hits,
+        held / (1 << 30),
     )
     return copies
 

@@ -380,6 +380,38 @@ class _PinnedPool:
 PINNED = _PinnedPool()
 
 
+class _RingPool:
+    """Device rings of the serving pipeline with the two streams that work on them, kept
+    between requests: a recovery fetches one payload as several ranges, again and again over
+    a job's life, and each request would otherwise allocate 3 x chunk_bytes of device memory
+    and two streams of its own.  A ring is allocated under its own gather stream, so taking
+    one never touches the training thread's stream."""
+
+    def __init__(self, keep: int = 8) -> None:
+        self._lock = threading.Lock()
+        self._free: List[Tuple[torch.Tensor, "torch.cuda.Stream", "torch.cuda.Stream"]] = []
+        self._keep = keep
+
+    def acquire(self, device: torch.device, nbytes: int):
+        with self._lock:
+            for i, (ring, _, _) in enumerate(self._free):
+                if ring.device == device and ring.numel() >= nbytes:
+                    return self._free.pop(i)
+        pack_stream, copy_stream = torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)
+        with torch.cuda.stream(pack_stream):
+            # every byte that is sent is gathered into the ring first: no need to clear it
+            ring = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        return ring, pack_stream, copy_stream
+
+    def release(self, item) -> None:
+        with self._lock:
+            if len(self._free) < self._keep:
+                self._free.append(item)
+
+
+RINGS = _RingPool()
+
+
 def split_range(total: int, part: int, parts: int) -> Tuple[int, int]:
     """Byte range [lo, hi) of ``part`` when a payload of ``total`` bytes is cut into
     ``parts`` ranges of (almost) equal size on 256-byte boundaries."""
@@ -415,9 +447,10 @@ def stream_packed(
     """Writes MAGIC | header length | header | payload bytes [lo, hi) to ``out`` without ever
     holding more than a few chunks: chunk k+2 is gathered on the device (one launch into a
     slot of a three-slot ring) while chunk k+1 crosses PCIe into pinned memory and chunk k is
-    written to ``out``.  Device memory: 3 x chunk_bytes; pinned memory: 3 x chunk_bytes.
-    The gather and the device-to-host copies run on two streams of their own, ordered after
-    ``after`` (an event recorded by whoever last wrote the state)."""
+    written to ``out``.  Device memory: 3 x chunk_bytes; pinned memory: 3 x chunk_bytes (both
+    pooled between calls).  The gather and the device-to-host copies run on two streams of
+    their own, ordered after ``after`` (an event recorded by whoever last wrote the state)
+    and after nothing else: the calling thread's current stream is not involved."""
     header = plan.header()
     out.write(MAGIC)
     out.write(struct.pack("<Q", len(header)))
@@ -432,14 +465,10 @@ def stream_packed(
     n_slots = 3
     chunk_bytes = max(ALIGN, min(chunk_bytes, -(-(hi - lo) // ALIGN) * ALIGN))
     starts = list(range(lo, hi, chunk_bytes))
-    ring = torch.zeros(n_slots * chunk_bytes, dtype=torch.uint8, device=device)
+    leased = RINGS.acquire(device, n_slots * chunk_bytes)
+    ring, pack_stream, copy_stream = leased
     slots = [ring[j * chunk_bytes : (j + 1) * chunk_bytes] for j in range(n_slots)]
     pinned = [PINNED.acquire(chunk_bytes) for _ in range(n_slots)]
-    pack_stream, copy_stream = torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)
-    # the ring was zeroed on the caller's stream
-    ready = torch.cuda.Event()
-    ready.record(torch.cuda.current_stream(device))
-    pack_stream.wait_event(ready)
     if after is not None:
         pack_stream.wait_event(after)
     packed = [torch.cuda.Event() for _ in starts]
@@ -474,6 +503,7 @@ def stream_packed(
         pack_stream.synchronize()
         for t in pinned:
             PINNED.release(t)
+        RINGS.release(leased)
 
 
 def write_packed(packed: PackedState, out: BinaryIO, chunk_bytes: int = DEFAULT_CHUNK_BYTES) -> None:
