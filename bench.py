@@ -876,7 +876,7 @@ def bench_ddp_hook(args) -> Dict[str, object]:
     (3 participate).  Everything runs on one stream, so GPU time is additive: the same backward
     is timed with the averaging hook and with ``manager.allreduce`` replaced by a stand-in that
     only returns the bucket, and HIP events around every ``manager.allreduce`` call give the
-    averaging kernels' own time."""
+    averaging kernels' own time (with the host kept ahead of the GPU, see ``backward``)."""
     from torch import nn
 
     from oracle import replica_sync as O
@@ -948,6 +948,15 @@ def bench_ddp_hook(args) -> Dict[str, object]:
 
     manager.allreduce = instrumented
 
+    # This synthetic backward is host-bound (hundreds of tiny launches), a real one is not: the
+    # host of a training step runs far ahead of the GPU.  To time GPU work rather than launch
+    # gaps, a plug of plain copies is enqueued first, long enough for the host to issue the
+    # whole backward while the GPU is still busy with the plug; everything behind it then
+    # executes back to back, and an event pair around a launch measures that launch alone.
+    plug_src = torch.empty(4 << 30, dtype=torch.uint8, device=dev)
+    plug_dst = torch.empty_like(plug_src)
+    plug_copies = [0]
+
     def backward(average: bool, record: bool = False) -> Tuple[float, float]:
         mode["average"], mode["record"] = average, record
         for p in model.parameters():
@@ -956,29 +965,41 @@ def bench_ddp_hook(args) -> Dict[str, object]:
         loss = ddp()
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(plug_copies[0]):
+            plug_dst.copy_(plug_src, non_blocking=True)
         t0 = time.perf_counter()
         a.record()
         loss.backward()
         b.record()
-        torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
         if not manager.should_commit():
             raise RuntimeError(f"the step did not commit: {manager.errored()!r}")
         return a.elapsed_time(b), wall
 
+    host_walls = []
     for _ in range(max(args.warmup, 2)):
-        backward(True)
+        host_walls.append(backward(True, record=True)[1])
         backward(False)
-    with_hook, without, kernels, walls = [], [], [], []
+    # one 4 GiB copy takes about 1.4 ms; cover the host's time for one backward three times
+    probe_a, probe_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    probe_a.record()
+    plug_dst.copy_(plug_src, non_blocking=True)
+    probe_b.record()
+    torch.cuda.synchronize()
+    plug_copies[0] = min(int(3.0 * min(host_walls) / probe_a.elapsed_time(probe_b)) + 1, 96)
+    with_hook, without, walls = [], [], []
     for _ in range(args.steps):
-        host_us.clear()
-        spans.clear()
-        gpu_ms, wall_ms = backward(True, record=True)
+        gpu_ms, wall_ms = backward(True)  # no events inside: they would sit between the launches
         with_hook.append(gpu_ms)
         walls.append(wall_ms)
-        kernels.append(sum(a.elapsed_time(b) for a, b in spans))
-        n_hooks, host_per_hook = len(spans), sum(host_us) / max(len(host_us), 1)
         without.append(backward(False)[0])
+    # one more pass, instrumented, for the host's time per hook call (its GPU figures are not used)
+    host_us.clear()
+    spans.clear()
+    backward(True, record=True)
+    n_hooks, host_per_hook = len(spans), sum(host_us) / max(len(host_us), 1)
+    in_situ = sum(a.elapsed_time(b) for a, b in spans)
     mean = lambda xs: sum(xs) / len(xs)
 
     # spot check of the last averaged backward against the checker: whole gradients of a few
@@ -1003,22 +1024,27 @@ def bench_ddp_hook(args) -> Dict[str, object]:
 
     hook_ms = mean(with_hook) - mean(without)
     out = base_line(args, "DDP gradient-bucket average elements/sec through the comm hook, Llama-3-8B bf16",
-                    n_elems / (mean(kernels) * 1e-3), "elements/s", mean(kernels), "bf16 storage, f32 accumulate",
+                    n_elems / (hook_ms * 1e-3), "elements/s", hook_ms, "bf16 storage, f32 accumulate",
                     {"workload": f"torch DistributedDataParallel(gradient_as_bucket_view=True) over the {len(shapes)} "
                                  f"Llama-3-8B bf16 parameters ({n_elems} elements), {n_hooks} buckets, comm hook = "
                                  "manager.allreduce(bucket.buffer()) on ProcessGroupLocalReplicas(world 4, one spare, "
-                                 "3 participate); one step = one real backward; ms_per_step is the sum of the "
-                                 "averaging kernels' time (HIP events around each manager.allreduce call)",
+                                 "3 participate); one step = one real backward; ms_per_step is the GPU time the "
+                                 "averaging hook adds to that backward (same backward with a pass-through hook "
+                                 "subtracted; one stream, host kept ahead of the GPU)",
                      "n_buckets": n_hooks, "n_elements": n_elems,
                      "output_check": f"gradients {picks} equal the CPU checker's bucket average bit for bit"})
-    out["roofline"] = roofline(n_elems * 2 * (n_active + 1), mean(kernels),
+    out["roofline"] = roofline(n_elems * 2 * (n_active + 1), hook_ms,
                                "mt_stream_kernel<BF16, ReduceAvgOp<1, 4>, FlatLocator>", n_hooks)
+    out["roofline"]["note"] = ("kernel_ms_per_step is the GPU time added to one backward by the 162 averaging "
+                               "launches, the gaps between them and their neighbours included; the kernels' own "
+                               "durations are in the rocprofv3 summary of this command")
     out["hook_seat"] = {
         "backward_gpu_ms_with_averaging_hook": mean(with_hook),
         "backward_gpu_ms_with_pass_through_hook": mean(without),
         "difference_ms": hook_ms,
-        "frac_of_peak_by_difference": n_elems * 2 * (n_active + 1) / (hook_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "backward_wall_ms_with_averaging_hook": mean(walls),
+        "event_spans_around_the_hook_calls_ms": in_situ,
+        "host_ms_to_issue_one_backward_with_averaging_hook": mean(walls),
+        "plug_copies_of_4GiB_ahead_of_each_backward": plug_copies[0],
         "host_us_per_hook": host_per_hook,
         "hooks_per_backward": n_hooks,
     }
