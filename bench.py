@@ -73,6 +73,9 @@ def parse_args() -> argparse.Namespace:
                          "and momentum allocated by the library's bank-group placement), no_placement "
                          "(the library allocates backup / momentum / pseudo-gradients without looking "
                          "at HBM bank groups)")
+    ap.add_argument("--placement-all", action="store_true",
+                    help="placement_llama3_8b_slice: every assignment of the streams to the three bank "
+                         "groups (up to relabelling the groups) instead of a selection")
     ap.add_argument("--model-copies", type=int, default=1,
                     help="DiLoCo workloads: the tensor list repeated this many times in one launch "
                          "(separates the fixed cost of a launch from its streaming rate)")
@@ -548,8 +551,7 @@ def bench_diloco_two_phase(args) -> Dict[str, object]:
     wl = workloads.make_diloco_workload(shapes, n_rep, dev)
     params = wl.replicas[0]  # live parameters are replica 0
     # backup, momentum and pseudo-gradients are the library's: allocated the way DiLoCo does
-    backup, bufs = hbm_placement.model_copies(params, 2)
-    grads = hbm_placement.model_copies(params, 1)[0]
+    backup, bufs, grads = hbm_placement.model_copies(params, 3)  # one search, as DiLoCo does
     ops.mt_copy(backup, wl.backup)
     ops.mt_copy(bufs, workloads.normal_tensors(shapes, 1e-3, 4000, dev))
     torch.cuda.synchronize()
@@ -602,6 +604,7 @@ def bench_placement(args) -> Dict[str, object]:
     n_params = sum(workloads.numel(sh) for _, sh in shapes)
     per_stream = sum(-(-workloads.numel(sh) * 4 // 256) * 256 for _, sh in shapes)
     pool = hbm_placement.GroupedPool(dev)
+    pool.limit = 280 << 30  # this workload wants all three groups, whatever that takes
     need = 5 * per_stream + (4 << 30)
     ok = pool.grow_until(lambda pl: len(pl.map.anchors) >= 3 and
                          all(pl.free_bytes(g) >= need for g in range(3)))
@@ -629,6 +632,16 @@ def bench_placement(args) -> Dict[str, object]:
     rows = []
     letters = "ABC"
     fused = ["AAAAA", "AABBB", "AABBA", "AACCA", "AABCA", "AAABA", "AAAAB", "AAABC", "AACAB", "ACACB"]
+    in_place = ["AAAA", "ABBB", "AABB", "AABC", "AABA", "ABAB", "ABCA"]
+    average = ["AAA", "ABB", "AAB", "ABA", "ABC"]
+    if args.placement_all:
+        # the first parameter stream (x0, or p where it is replica 0) fixed in group A: the
+        # three groups are interchangeable
+        import itertools
+
+        fused = ["A" + "".join(t) for t in itertools.product(letters, repeat=4)]
+        in_place = ["".join((t[0], "A", t[1], t[2])) for t in itertools.product(letters, repeat=3)]
+        average = ["".join((t[0], "A", t[1])) for t in itertools.product(letters, repeat=2)]
     for lay in fused:  # streams x0 x1 b buf p
         pool.reset()
         x0, x1, b, buf, p = (column(letters.index(c), s) for c, s in zip(lay, (0.02, 0.02, 0.02, 0.0, 0.0)))
@@ -636,14 +649,14 @@ def bench_placement(args) -> Dict[str, object]:
         rows.append({"kernel": "fused DiLoCo, separate output", "streams": "x0 x1 b buf p", "groups": lay,
                      "kernel_ms": ms, "frac": n_params * 28 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
         del x0, x1, b, buf, p
-    for lay in ["AAAA", "ABBB", "AABB", "AABC", "AABA", "ABAB", "ABCA"]:  # streams x1 p b buf (p is replica 0)
+    for lay in in_place:  # streams x1 p b buf (p is replica 0)
         pool.reset()
         x1, p, b, buf = (column(letters.index(c), s) for c, s in zip(lay, (0.02, 0.02, 0.02, 0.0)))
         ms = measure(lambda: ops.mt_diloco_outer(p, b, buf, [p, x1], sgd, False))
         rows.append({"kernel": "fused DiLoCo, parameters in place", "streams": "x1 p b buf", "groups": lay,
                      "kernel_ms": ms, "frac": n_params * 28 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
         del x1, p, b, buf
-    for lay in ["AAA", "ABB", "AAB", "ABA", "ABC"]:  # streams x1 p b
+    for lay in average:  # streams x1 p b
         pool.reset()
         x1, p, b = (column(letters.index(c), 0.02) for c in lay)
         ms = measure(lambda: ops.mt_reduce_avg([p, b], [p, x1]))

@@ -95,7 +95,9 @@ class _IPv6HTTPServer(ThreadingHTTPServer):
 
 
 def _default_streams() -> int:
-    return max(1, int(os.environ.get("TORCHFT_AMD_CHECKPOINT_STREAMS", "4")))
+    # one TCP stream carries what two copies through the kernel allow one core (8-9 GB/s over
+    # loopback); eight of them reach 30 GB/s between two processes, four 26 GB/s
+    return max(1, int(os.environ.get("TORCHFT_AMD_CHECKPOINT_STREAMS", "8")))
 
 
 class CheckpointServer(CheckpointTransport[T]):
