@@ -73,6 +73,11 @@ def parse_args() -> argparse.Namespace:
                          "and momentum allocated by the library's bank-group placement), no_placement "
                          "(the library allocates backup / momentum / pseudo-gradients without looking "
                          "at HBM bank groups)")
+    ap.add_argument("--launch-variant", default="",
+                    help="route the launches through the tuning build of the library with this launch-shape "
+                         "override (bits 0-3 accesses per lane: 1, 2, 4; bit 4 plain instead of non-temporal "
+                         "accesses; bits 8-11 log2 of the per-XCD run + 1; bits 12-15 dynamic LDS per workgroup "
+                         "in units of 8 KiB + 1, e.g. 0x1000 = no residency cap, 0x9000 = 64 KiB); for sweeps")
     ap.add_argument("--placement-all", action="store_true",
                     help="placement_llama3_8b_slice: every assignment of the streams to the three bank "
                          "groups (up to relabelling the groups) instead of a selection")
@@ -1342,6 +1347,15 @@ def main() -> int:
         time.sleep(args.settle_seconds)  # before anything is allocated on the device
     torch.cuda.set_device(0)
     from torchft_amd import ops
+
+    if args.launch_variant:
+        import ctypes
+
+        from torchft_amd import _build, _native
+
+        tuning = _native.load(_build.TUNING_LIB_PATH, {"tft_set_launch_variant": (None, [ctypes.c_uint32])})
+        _native._lib = tuning
+        tuning.tft_set_launch_variant(int(args.launch_variant, 0))  # thread-local: this thread launches
 
     if args.calibration_copy and not args.workload.startswith("diloco_llama3_8b"):
         # reference point for hardware-counter runs: a plain copy of exactly 8 GiB

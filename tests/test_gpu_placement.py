@@ -231,3 +231,38 @@ def test_two_replicas_constructing_at_once_take_turns(device):
         for i, p in enumerate(models[k].parameters()):
             assert_bits_equal(p.data, want["params"][i], f"replica {k} params[{i}]")
         manager.shutdown(wait=False)
+
+
+def test_momentum_set_aside_for_a_fused_step_is_released_when_the_step_is_not_fused(device):
+    """The outer momentum is allocated with the backup when the outer optimizer looks like a
+    fusable SGD.  If it then is not (here: a tensor learning rate), the optimizer's own step()
+    runs and creates its own state: the buffers set aside must not stay allocated."""
+    torch.manual_seed(0)
+    model = Wide().to(device)
+    peer = [p.data + 1e-3 for p in model.parameters()]
+    index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]])
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=torch.tensor(0.7), momentum=0.9, nesterov=True)
+    ctx = DiLoCo(manager, model, inner, outer, sync_every=10 ** 9)
+    if ctx._placed_momentum is None:
+        pytest.skip("no bank-group structure found: is this an MI355X?")
+    set_aside = ctx._placed_momentum[0].data_ptr()
+    before = torch.cuda.memory_allocated(device)
+    with ctx:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1e-3)
+        ctx.sync()
+    torch.cuda.synchronize()
+    assert ctx._placed_momentum is None
+    # the copies fill blocks of their own, so most of the 1.25 GiB set aside is free again
+    # (the optimizer's own buffers, as large, have been allocated meanwhile)
+    assert torch.cuda.memory_allocated(device) - before < (1 << 30)
+    # the optimizer made its own buffers; ours are not among them
+    assert all(outer.state[p]["momentum_buffer"].data_ptr() != set_aside for p in model.parameters())
+    for p, b in zip(model.parameters(), ctx._backup_parameters.values()):
+        assert_bits_equal(p.data, b)
+    manager.shutdown(wait=False)

@@ -558,10 +558,10 @@ def _allocate_apart(
         by_group: Dict[int, List[_Block]] = {}
         for b in pl.blocks:
             by_group.setdefault(b.group, []).append(b)
-        for i in order:
-            if not sizes[i]:
-                continue
-            for _ in range(n_copies):
+        for _ in range(n_copies):  # same order as the hand-out below
+            for i in order:
+                if not sizes[i]:
+                    continue
                 for b in by_group.get(wanted[i], ()):
                     start = -(-cursors[id(b)] // ALIGN) * ALIGN
                     if start + sizes[i] <= b.storage.numel():
@@ -575,13 +575,16 @@ def _allocate_apart(
     n_groups = len(pool.map.anchors)
     placed: Dict[Tuple[int, int], Optional[torch.Tensor]] = {}
     misplaced = 0
-    for i in order:
-        prefer = wanted[i]
-        own = groups[i]
-        others = [g for g in range(n_groups) if g != prefer and g != own]
-        if own is not None and own != prefer:
-            others.append(own)  # the tensor's own group last
-        for k in range(n_copies):
+    # copy by copy, so that each copy fills blocks of its own (up to one shared block where
+    # two copies meet): a copy its owner drops then gives its memory back, instead of every
+    # block staying pinned by the other copies' tensors
+    for k in range(n_copies):
+        for i in order:
+            prefer = wanted[i]
+            own = groups[i]
+            others = [g for g in range(n_groups) if g != prefer and g != own]
+            if own is not None and own != prefer:
+                others.append(own)  # the tensor's own group last
             raw = pool.take(sizes[i], [prefer]) if sizes[i] else None
             if raw is None and sizes[i]:
                 raw = pool.take(sizes[i], others)
