@@ -11,12 +11,13 @@
  *     device pointer, everything else is host memory;
  *   - return 0 on success, a negative tft_status on error; tft_last_error()
  *     returns a thread-local message for the last failing call on this thread;
- *   - the library never allocates device memory, never synchronises and keeps
- *     no mutable global state (the error string is thread-local): each call
- *     validates its arguments on the host and enqueues exactly one kernel on the
- *     caller's hipStream_t (passed as void*; NULL is the legacy default stream).
- *     The one exception is tft_mt_diloco_outer_noalloc, which enqueues a few
- *     kernels and uses a fixed device array owned by the library;
+ *   - the library never allocates device memory and never synchronises: each
+ *     call validates its arguments on the host and enqueues exactly one kernel on
+ *     the caller's hipStream_t (passed as void*; NULL is the legacy default
+ *     stream).  Mutable state: the error string (thread-local), and for
+ *     tft_mt_diloco_outer_noalloc alone a fixed device array owned by the library
+ *     together with its per-device address (that entry enqueues a few kernels);
+ *     nothing else is kept between calls;
  *   - re-entrant: may be called concurrently from the training thread, the
  *     autograd thread (DDP comm hook) and the checkpoint thread.
  *
