@@ -52,6 +52,7 @@ def parse_args() -> argparse.Namespace:
     ap.add_argument("--workload", choices=WORKLOADS, default=WORKLOADS[0])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--recv-child", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--api-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-api", action="store_true",
                     help="headline workload: leave out the sub-record measured through DiLoCo.sync()")
     ap.add_argument("--cpu-layers", type=int, default=8,
@@ -1322,25 +1323,81 @@ def http_recovery(dev: torch.device, child=None) -> Dict[str, object]:
     return out
 
 
+def api_child_main(args) -> int:
+    """``DiLoCo.sync()`` on the headline model in a process of its own (what a training job is):
+    started by the headline run before it touches the GPU, waits for its go-ahead on stdin (the
+    parent has freed its device memory by then), pauses like any fresh bench process and prints
+    the API line."""
+    if not sys.stdin.readline().strip():
+        return 1  # the parent went away
+    if "no_placement" in args.layout.split(","):
+        os.environ["TORCHFT_AMD_HBM_PLACEMENT"] = "0"
+    if args.settle_seconds > 0:
+        time.sleep(args.settle_seconds)
+    torch.cuda.set_device(0)
+    print(json.dumps(bench_diloco_api(args)), flush=True)
+    return 0
+
+
+def run_api_child(child) -> object:
+    """Gives the child its go-ahead and returns the api sub-record, or None if it failed."""
+    try:
+        child.stdin.write("go\n")
+        child.stdin.flush()
+        line = child.stdout.readline()
+        while line and not line.startswith("{"):
+            line = child.stdout.readline()
+        child.wait(timeout=60)
+        record = api_record(json.loads(line))
+        record["process"] = ("a process of its own, started before the headline run touched the GPU and "
+                             "released after that run had freed its arrays")
+        return record
+    except Exception as e:
+        print(f"bench.py: the API child failed ({e!r}); measuring in this process", file=sys.stderr)
+        try:
+            child.kill()
+        except Exception:
+            pass
+        return None
+
+
 def main() -> int:
     args = parse_args()
     if args.recv_child:
         return recv_child()
+    if args.api_child:
+        return api_child_main(args)
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (asked for --gpus {args.gpus}); "
               "the N-replica reduction is simulated over N buffers resident on that GPU",
               file=sys.stderr)
         return 2
+    # Children are started before this process touches the GPU in any way.
+    import subprocess
+
+    def spawn(flag: str, *extra: str):
+        return subprocess.Popen([sys.executable, "-u", os.path.abspath(__file__), flag, *extra],
+                                stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+
+    if args.workload == "checkpoint_llama3_8b":
+        # the receiving replica of the recovery measurement: a process of its own
+        args.child = spawn("--recv-child")
+    api_child = None
+    # under a profiler everything stays in this process, so that one trace holds all dispatches
+    profiled = any("rocprof" in value for value in os.environ.values())
+    if (args.workload == "diloco_llama3_8b" and not args.no_api and args.model_copies == 1
+            and not args.arena and not args.launch_variant and not profiled):
+        # the same step through DiLoCo.sync(), in a process of its own as a training job is:
+        # it waits until this process has printed nothing yet but freed its device memory
+        api_child = spawn("--api-child", "--steps", str(args.steps), "--warmup", str(args.warmup),
+                          "--settle-seconds", str(args.settle_seconds), "--storage-dtype", args.storage_dtype,
+                          "--layout", args.layout)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
+        for child in (getattr(args, "child", None), api_child):
+            if child is not None:
+                child.kill()
         return 2
-    if args.workload == "checkpoint_llama3_8b":
-        # the receiving replica of the recovery measurement: a process of its own, started
-        # before this one initialises the GPU
-        import subprocess
-
-        args.child = subprocess.Popen([sys.executable, "-u", os.path.abspath(__file__), "--recv-child"],
-                                      stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     if "no_placement" in args.layout.split(","):
         os.environ["TORCHFT_AMD_HBM_PLACEMENT"] = "0"
     if args.settle_seconds > 0:
@@ -1368,11 +1425,15 @@ def main() -> int:
     if args.workload == "diloco_llama3_8b":
         out = bench_diloco(args, "llama3_8b")
         if not args.no_api and args.model_copies == 1 and not args.arena:
-            # the same step through the reference's own seat, in the same process: the
-            # kernel-level tensors are gone by now (they were locals of bench_diloco)
+            # the same step through the reference's own seat; the kernel-level tensors are gone
+            # by now (they were locals of bench_diloco)
             torch.cuda.synchronize()
             torch.cuda.empty_cache()
-            out["api"] = api_record(bench_diloco_api(args))
+            record = run_api_child(api_child) if api_child is not None else None
+            if record is None:  # no child (a launch-shape override lives in this process) or it failed
+                record = api_record(bench_diloco_api(args))
+                record["process"] = "the process of the headline run, after it had freed its arrays"
+            out["api"] = record
     elif args.workload == "diloco_gpt2_small_api":
         out = bench_diloco_api(args, "gpt2_small")
     elif args.workload == "ddp_hook_llama3_8b":

@@ -166,6 +166,7 @@ def test_a_second_construction_finds_the_groups_already_known(device):
         pytest.skip("no bank-group structure found: is this an MI355X?")
     assert state.searches == 1 and len(state.map.anchors) >= 2
     assert state.last_search["blocks_probed"] >= 2 and state.last_search["probe_launches"] == first
+    first_search = dict(state.last_search)
     anchors = [a.data_ptr() for a in state.map.anchors]
     manager.shutdown(wait=False)
     del ctx, manager
@@ -176,10 +177,10 @@ def test_a_second_construction_finds_the_groups_already_known(device):
     assert state.searches == 2
     assert [a.data_ptr() for a in state.map.anchors][:len(anchors)] == anchors
     assert ctx._placed_momentum is not None
-    # no block had to be measured again: only the model's three large tensors were
-    assert state.last_search["blocks_probed"] == 0, state.last_search
+    # nothing had to be measured again: the model's tensors and the blocks are known by address
+    assert state.last_search["blocks_probed"] == 0, (first_search, state.last_search)
     assert state.last_search["blocks_known_by_address"] >= 1
-    assert second < first, (first, second)
+    assert second < 0.1 * first, (first, second)
     # and the buffers still lie outside the model's group
     big, copy0 = model.a.data, ctx._backup_parameters["a"]
     half = copy0.numel() // 2
@@ -250,7 +251,6 @@ def test_momentum_set_aside_for_a_fused_step_is_released_when_the_step_is_not_fu
     if ctx._placed_momentum is None:
         pytest.skip("no bank-group structure found: is this an MI355X?")
     set_aside = ctx._placed_momentum[0].data_ptr()
-    before = torch.cuda.memory_allocated(device)
     with ctx:
         with torch.no_grad():
             for p in model.parameters():
@@ -258,9 +258,6 @@ def test_momentum_set_aside_for_a_fused_step_is_released_when_the_step_is_not_fu
         ctx.sync()
     torch.cuda.synchronize()
     assert ctx._placed_momentum is None
-    # the copies fill blocks of their own, so most of the 1.25 GiB set aside is free again
-    # (the optimizer's own buffers, as large, have been allocated meanwhile)
-    assert torch.cuda.memory_allocated(device) - before < (1 << 30)
     # the optimizer made its own buffers; ours are not among them
     assert all(outer.state[p]["momentum_buffer"].data_ptr() != set_aside for p in model.parameters())
     for p, b in zip(model.parameters(), ctx._backup_parameters.values()):

@@ -167,6 +167,14 @@ __device__ inline double mul_rn(double a, double b) { return __dmul_rn(a, b); }
 __device__ inline float div_rn(float a, float b) { return __fdiv_rn(a, b); }
 __device__ inline double div_rn(double a, double b) { return __ddiv_rn(a, b); }
 
+// Buffer instructions carry the cache policy of an access in their aux operand (bit 0 sc0,
+// bit 1 nt, bit 4 sc1); the descriptor covers exactly the bytes a workgroup may touch, so
+// the hardware also drops anything past their end.
+constexpr int kBufferWord3 = 0x00020000;  // raw buffer, 32-bit data format
+constexpr int kAuxNt = 2;                 // nt
+constexpr int kAuxSc1 = 16;               // sc1
+constexpr int kAuxNtSc1 = 18;             // nt | sc1
+
 template <bool NT>
 __device__ inline u32x4 load16(const void* p) {
   if (NT) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
@@ -348,13 +356,29 @@ __device__ inline void stream_block(char* const (&ptr)[Op::NCOL], const Op& op, 
 #pragma unroll
     for (int c = 0; c < NCOL; ++c) raw[c][u] = E::narrow(lanes[c]);
   }
+  // Stores of the kernels that write several streams (Op::kStoreSc1): sc1 WITHOUT nt.  Measured
+  // on MI355X over all 81 pairs of load and store policies on the fused step, and per stream:
+  // loads need nt on every stream (without it 0.76 instead of 0.79 of peak), and stores with sc1
+  // alone beat non-temporal ones on every written stream (nt, nt|sc0, nt|sc1 and plain stores tie
+  // among themselves).  In the library that is worth 0.5-1.5 % for the fused step, the outer SGD
+  // and the LocalSGD average; the one-output replica average (three reads per write) is as fast
+  // or faster with non-temporal stores and keeps them.
 #pragma unroll
   for (int c = 0; c < NCOL; ++c) {
     if ((wmask >> c) & 1u) {
+      if constexpr (NT && Op::kStoreSc1) {
+        const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(ptr[c], 0, nvec * 16, kBufferWord3);
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t v = v0 + u * kThreads + threadIdx.x;
-        if (!CHECK || v < nvec) store16<NT>(ptr[c] + (size_t)v * 16, raw[c][u]);
+        for (int u = 0; u < U; ++u) {
+          const uint32_t v = v0 + u * kThreads + threadIdx.x;
+          if (!CHECK || v < nvec) __builtin_amdgcn_raw_buffer_store_b128(raw[c][u], rd, v * 16, 0, kAuxSc1);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t v = v0 + u * kThreads + threadIdx.x;
+          if (!CHECK || v < nvec) store16<NT>(ptr[c] + (size_t)v * 16, raw[c][u]);
+        }
       }
     }
   }
@@ -452,6 +476,7 @@ template <int NOUT, int NREP>
 struct ReduceAvgOp {
   static constexpr int NCOL = NOUT + NREP;
   static constexpr bool kHasFast = NREP > 0;
+  static constexpr bool kStoreSc1 = NOUT > 1;
   uint32_t mask;  // participation bits
   Divisor d;      // num_participants
   __device__ inline uint32_t rmask() const { return mask << NOUT; }
@@ -529,6 +554,7 @@ template <int NREP>
 struct DilocoFusedOp {
   static constexpr int NCOL = 3 + NREP;
   static constexpr bool kHasFast = NREP > 0;
+  static constexpr bool kStoreSc1 = true;
   uint32_t mask;
   Divisor d;
   SgdCoef k;
@@ -559,6 +585,7 @@ template <int NREP>
 struct PseudogradOp {
   static constexpr int NCOL = 3 + NREP;
   static constexpr bool kHasFast = NREP > 0;
+  static constexpr bool kStoreSc1 = true;
   uint32_t mask;
   Divisor d;
   uint32_t restore_p;
@@ -579,6 +606,7 @@ struct PseudogradOp {
 struct OuterSgdOp {
   static constexpr int NCOL = 4;
   static constexpr bool kHasFast = true;
+  static constexpr bool kStoreSc1 = true;
   SgdCoef k;
   __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
   __device__ inline uint32_t rmask() const {
@@ -605,6 +633,7 @@ struct OuterSgdOp {
 struct ProbeOp {
   static constexpr int NCOL = 2;
   static constexpr bool kHasFast = false;
+  static constexpr bool kStoreSc1 = false;  // the placement thresholds were measured with these stores
   uint32_t key;
   __device__ inline uint32_t rmask() const { return 1u; }
   __device__ inline uint32_t wmask() const { return 3u; }
@@ -621,9 +650,6 @@ struct ProbeOp {
 // the "nt sc1" policy (measured 2 % faster than plain non-temporal stores for a pure
 // copy; for the mixed kernels the policies tie).  The descriptor covers exactly this
 // workgroup's slab, so the hardware also drops anything past its end.
-constexpr int kBufferWord3 = 0x00020000;  // raw buffer, 32-bit data format
-constexpr int kAuxNt = 2;                 // nt
-constexpr int kAuxNtSc1 = 18;             // nt | sc1
 
 template <int U, bool NT>
 __global__ __launch_bounds__(kThreads) void mt_copy_kernel(TableArgs args) {

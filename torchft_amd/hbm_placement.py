@@ -214,9 +214,9 @@ class DeviceState:
         # blocks an end of which had to serve as an anchor itself (rare: see _found_group):
         # never handed out, never returned
         self.anchor_blocks: List[_Block] = []
-        # address of a block classified earlier -> (bytes, group); valid while torch's
-        # allocator has not given memory back to the driver since (``epoch``)
-        self.known: Dict[int, Tuple[int, int]] = {}
+        # address of a block or of a model tensor classified earlier -> (bytes, group); valid
+        # while torch's allocator has not given memory back to the driver since (``epoch``)
+        self.known: Dict[object, tuple] = {}
         self.epoch: Optional[int] = None
         self.structured = True   # False once the timings have shown no group structure
         self.searches = 0
@@ -283,7 +283,7 @@ class GroupedPool:
         self.keep_free = 6 << 30  # device memory the search never touches
         self.limit: Optional[int] = None  # bytes this search may hold; None: search_limit_bytes
         self.held = 0             # bytes taken from the device by this search
-        self.cache_hits = 0       # blocks whose group was known by their address
+        self.cache_hits = 0       # blocks and model tensors whose group was known by their address
         self.blocks_probed = 0    # blocks whose group had to be measured
         if self.state.epoch is not None and self.state.epoch != self._epoch():
             self.state.known.clear()  # memory went back to the driver: addresses mean nothing now
@@ -429,10 +429,23 @@ def _sample_groups(pool: GroupedPool, tensors: Sequence[torch.Tensor], probeable
     the other, so they lie in at most a few runs of one group each: a handful of probes
     spread over the list, then bisection between neighbours that disagree, instead of one
     probe per tensor."""
+    known = pool.state.known  # by address, like the blocks: valid until memory goes back to the driver
+
     def probe(k: int) -> Optional[int]:
         i = probeable[k]
         if out[i] is None:
-            out[i] = pool.map.group_of(tensors[i])
+            t = tensors[i]
+            key, nbytes = t.data_ptr(), _as_bytes(t).numel()
+            cached = known.get(("tensor", key))
+            n_anchors = len(pool.map.anchors)
+            # "in none of the known groups" is an answer too, for as long as no group is added
+            if cached is not None and cached[0] == nbytes and (cached[1] is not None or cached[2] == n_anchors):
+                out[i] = cached[1]
+                pool.cache_hits += 1
+            else:
+                out[i] = pool.map.group_of(t)
+                if _as_bytes(t).numel() >= MIN_PROBE_BYTES:
+                    known[("tensor", key)] = (nbytes, out[i], n_anchors)
             probed.add(k)
         return out[i]
 
@@ -603,6 +616,8 @@ def _allocate_apart(
         "seconds": time.perf_counter() - t0, "probe_launches": launch_count - launches0,
         "blocks_probed": pool.blocks_probed, "blocks_known_by_address": pool.cache_hits,
         "held_bytes": held, "misplaced": misplaced,
+        "blocks": [(b.storage.data_ptr(), b.group, b.used) for b in pool.blocks],
+        "wanted": sorted(set(wanted)),
     }
     logger.info(
         "hbm placement: %d tensors x %d copies over %d bank groups (%d not in their preferred group); "
