@@ -1179,3 +1179,171 @@ def test_local_sgd_fused_applies_recovered_state_with_asynchronous_quorum(cpu_op
         for p, q in zip(model.parameters(), peers[0].parameters()):
             assert_bits_equal(p.data, q.data)
     manager.shutdown(wait=False)
+
+
+# ---------------------------------------------------------------------------
+# What a wrapper keeps between syncs, and what makes it look again
+# ---------------------------------------------------------------------------
+
+def _stable_world(model: nn.Module, n: int):
+    """Peer models whose buffers never move, a lookup that counts its calls, and a process
+    group that has been told so (``peers_are_stable``)."""
+    import copy
+
+    peers = [copy.deepcopy(model) for _ in range(n - 1)]
+    calls = []
+
+    def lookup(t):
+        calls.append(t.data_ptr())
+        for k, p in enumerate(model.parameters()):
+            if p.data.data_ptr() == t.data_ptr():
+                return [list(peer.parameters())[k].data for peer in peers]
+        raise KeyError("unknown tensor")
+
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=n, peer_lookup=lookup, peers_are_stable=True)
+    return peers, pg, calls
+
+
+def _checked_diloco_sync(diloco, model, peers, outer, state, lr=0.7):
+    """One sync, compared with the checker; ``state`` carries (backup, momentum) along."""
+    with torch.no_grad():
+        for p in model.parameters():
+            p.add_(1e-3 * torch.randn_like(p))
+    local = [p.data.clone() for p in model.parameters()]
+    want = O.diloco_perform_sync(
+        [local] + [[q.data.clone() for q in peer.parameters()] for peer in peers],
+        state["backup"], state["bufs"], [True] * (len(peers) + 1), len(peers) + 1, True,
+        lr=lr, momentum=0.9, nesterov=True)
+    diloco.sync()
+    for p, w in zip(model.parameters(), want["params"]):
+        assert_bits_equal(p.data, w)
+    for b_, w in zip(diloco._backup_parameters.values(), want["backup"]):
+        assert_bits_equal(b_, w)
+    for p, w in zip(model.parameters(), want["momentum"]):
+        assert_bits_equal(outer.state[p]["momentum_buffer"], w)
+    state["backup"], state["bufs"] = want["backup"], want["momentum"]
+
+
+def test_diloco_keeps_its_prepared_sync_and_notices_every_change(cpu_ops):
+    """Steady state: no peer lookups, no new tensor lists, the same prepared launch.  Each thing a
+    user may change between syncs - ``p.data``, ``_backup_parameters``, the learning rate, the
+    optimizer's state, the peers - is noticed, and the results stay the checker's."""
+    torch.manual_seed(0)
+    model = SimpleModel()
+    peers, pg, lookups = _stable_world(model, 2)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    n = len(list(model.parameters()))
+    state = {"backup": [p.data.clone() for p in model.parameters()], "bufs": None}
+    with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
+        _checked_diloco_sync(diloco, model, peers, outer, state)      # first step: creates momentum
+        _checked_diloco_sync(diloco, model, peers, outer, state)      # steady state: prepared anew once
+        assert len(lookups) == n                                      # asked once per tensor, ever
+        kept, bound, plan = diloco._launches["fused"], diloco._bound, diloco._plan
+        for _ in range(2):
+            _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert len(lookups) == n
+        assert diloco._launches["fused"] is kept and diloco._bound is bound and diloco._plan is plan
+
+        # the learning rate moves (a scheduler): new plan, same tensors
+        outer.param_groups[0]["lr"] = 0.35
+        _checked_diloco_sync(diloco, model, peers, outer, state, lr=0.35)
+        assert diloco._plan is not plan and diloco._bound is bound and len(lookups) == n
+        outer.param_groups[0]["lr"] = 0.7
+
+        # a parameter's storage is replaced (model.to(), a load that rebinds .data)
+        first = next(model.parameters())
+        first.data = first.data.clone()
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert diloco._bound is not bound and len(lookups) == 2 * n   # peers looked up again
+        bound = diloco._bound
+
+        # the user's load_state_dict assigns a new backup dict (torchft/manager_integ_test.py:279)
+        diloco._backup_parameters = {k: v.clone() for k, v in diloco._backup_parameters.items()}
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert diloco._bound is not bound
+        bound = diloco._bound
+
+        # the outer optimizer's state is replaced (load_state_dict after healing)
+        saved = copy_state = outer.state_dict()
+        outer.load_state_dict(copy_state)
+        state["bufs"] = [outer.state[p]["momentum_buffer"].clone() for p in model.parameters()]
+        plan = diloco._plan
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert diloco._plan is not plan
+
+        # a momentum buffer is swapped inside the state
+        p0 = next(model.parameters())
+        outer.state[p0]["momentum_buffer"] = outer.state[p0]["momentum_buffer"].clone()
+        plan = diloco._plan
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert diloco._plan is not plan
+
+        # the peers move and say so
+        for q in peers[0].parameters():
+            q.data = q.data.clone()
+        pg.invalidate_peers()
+        before = len(lookups)
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        assert len(lookups) == before + n
+    manager.shutdown(wait=False)
+
+
+def test_peer_lookups_are_repeated_unless_declared_stable(cpu_ops):
+    torch.manual_seed(0)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 2)
+    seen = []
+
+    def counting(t):
+        seen.append(1)
+        return lookup(t)
+
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=counting)
+    assert pg.peers_generation() is None          # a callback may answer differently next time
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    n = len(list(model.parameters()))
+    with LocalSGD(manager, model, inner, sync_every=10 ** 9) as lsgd:
+        for k in range(3):
+            lsgd.sync()
+            assert len(seen) == (k + 1) * n
+    # registered peers only change through the group: a generation, and no repeated look-ups
+    pg2 = ProcessGroupLocalReplicas(rank=0, world_size=2)
+    t, peer = torch.zeros(4), torch.ones(4)
+    g0 = pg2.peers_generation()
+    pg2.register_peers(t, [peer])
+    assert pg2.peers_generation() == g0 + 1
+    pg2.set_peer_participating([False])
+    assert pg2.peers_generation() == g0 + 2
+    manager.shutdown(wait=False)
+
+
+def test_local_sgd_keeps_its_prepared_average(cpu_ops):
+    torch.manual_seed(0)
+    model = SimpleModel()
+    peers, pg, lookups = _stable_world(model, 3)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1,
+                      use_async_quorum=False, quorum_client=StaticQuorum(0, 3))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    n = len(list(model.parameters()))
+    with LocalSGD(manager, model, inner, sync_every=10 ** 9) as lsgd:
+        backup = [b.clone() for b in lsgd._backup_parameters.values()]
+        for k in range(3):
+            with torch.no_grad():
+                for p in model.parameters():
+                    p.add_(1e-3 * torch.randn_like(p))
+            reps = [[p.data.clone() for p in model.parameters()]] + [
+                [q.data.clone() for q in peer.parameters()] for peer in peers]
+            want = O.localsgd_perform_sync(reps, backup, [True] * 3, 3, True)
+            lsgd.sync()
+            for p, w in zip(model.parameters(), want["params"]):
+                assert_bits_equal(p.data, w)
+            backup = want["backup"]
+            if k == 0:
+                kept = lsgd._launches["average"]
+        assert lsgd._launches["average"] is kept and len(lookups) == n
+    manager.shutdown(wait=False)
