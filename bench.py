@@ -546,8 +546,10 @@ def bench_localsgd_api(args) -> Dict[str, object]:
 
 def bench_diloco_two_phase(args) -> Dict[str, object]:
     """The two-phase form used when the commit decision must come between reduction and
-    update: phase 1 (pseudo-gradient average + restore, in place on replica 0) and phase 2
-    (outer SGD + backup refresh), each one launch, timed separately."""
+    update: phase 1 (pseudo-gradient average, in place on replica 0) and phase 2 (outer SGD +
+    backup refresh), each one launch, timed separately.  Phase 1 leaves the parameters alone,
+    as DiLoCo.sync() does with a fusable SGD (phase 2 overwrites them without reading them);
+    the form that also restores them, used before any other optimizer, is timed beside it."""
     from torchft_amd import ops, workloads
 
     dev = torch.device("cuda", 0)
@@ -564,19 +566,25 @@ def bench_diloco_two_phase(args) -> Dict[str, object]:
     wl.backup = backup
     torch.cuda.empty_cache()
     sgd = ops.OuterSGD(lr=LR, momentum=MOMENTUM, nesterov=True)
-    t1 = ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, True)
+    t1 = ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, False)
     t2 = ops.mt_outer_sgd(params, wl.backup, bufs, grads, sgd, False)
     pristine = [t.clone() for t in wl.backup]  # phase 2 moves the backup: put it back per step
     torch.cuda.synchronize()
     n_params = wl.n_params
-    e = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    e = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
     for i in range(args.warmup + args.steps):
         k = i - args.warmup
         ops.mt_copy(wl.backup, pristine)
         ops.mt_copy(params, wl.replicas[1])  # some drift to average
         if k >= 0:
-            e[k][0].record()
+            e[k][3].record()
         ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, True, table=t1)
+        if k >= 0:
+            e[k][4].record()
+        ops.mt_copy(params, wl.replicas[1])
+        if k >= 0:
+            e[k][0].record()
+        ops.mt_pseudograd_avg(grads, params, wl.backup, wl.replicas, False, table=t1)
         if k >= 0:
             e[k][1].record()
         ops.mt_outer_sgd(params, wl.backup, bufs, grads, sgd, False, table=t2)
@@ -585,16 +593,19 @@ def bench_diloco_two_phase(args) -> Dict[str, object]:
     torch.cuda.synchronize()
     p1 = sum(a[0].elapsed_time(a[1]) for a in e) / args.steps
     p2 = sum(a[1].elapsed_time(a[2]) for a in e) / args.steps
+    p1r = sum(a[3].elapsed_time(a[4]) for a in e) / args.steps
     out = base_line(args, "two-phase DiLoCo sync params/sec, Llama-3-8B", n_params / ((p1 + p2) * 1e-3),
                     "params/s", p1 + p2, "f32",
-                    {"workload": "DiLoCo sync in two launches (pseudo-gradient average + restore, then outer "
-                                 "SGD + backup refresh), Llama-3-8B fp32, 2 replicas, in place on replica 0; "
+                    {"workload": "DiLoCo sync in two launches (pseudo-gradient average, then outer SGD + "
+                                 "backup refresh), Llama-3-8B fp32, 2 replicas, in place on replica 0; "
                                  "ms_per_step is the sum of the two kernels (the state reset between steps "
                                  "is not counted)",
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": n_rep})
-    # phase 1: read x0, x1, b; write g, p.  phase 2: read g, b, buf; write p, b, buf.
-    out["roofline"] = roofline(n_params * 20, p1, "mt_stream_kernel<F32, PseudogradOp<2>>")
+    # phase 1: read x0, x1, b; write g (and p where it restores).
+    # phase 2: read g, b, buf; write p, b, buf.
+    out["roofline"] = roofline(n_params * 16, p1, "mt_stream_kernel<F32, PseudogradOp<2>>")
     out["phase2"] = roofline(n_params * 24, p2, "mt_stream_kernel<F32, OuterSgdOp>")
+    out["phase1_with_restore"] = roofline(n_params * 20, p1r, "mt_stream_kernel<F32, PseudogradOp<2>>")
     return out
 
 

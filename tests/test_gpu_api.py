@@ -329,6 +329,27 @@ def test_diloco_fused_local_replicas(device):
     m.shutdown(wait=False)
 
 
+def test_diloco_two_launches_when_the_reduction_may_fail_late(device):
+    """A group whose reduction can fail after the launch takes the vote between the two
+    launches: pseudo-gradient average first (the parameters are left alone when the outer
+    SGD is fusable), then outer step (commit) or restore (no commit)."""
+    flag = [True]
+
+    def factory(lookup):
+        pg = ProcessGroupLocalReplicas(rank=0, world_size=3, peer_lookup=lookup)
+        pg.fails_only_at_launch = False
+
+        class Vote(StaticQuorum):
+            def should_commit(self, rank, step, should_commit, timeout):
+                return should_commit and flag[0]
+
+        return Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, use_async_quorum=False, quorum_client=Vote(0, 3)), flag
+
+    m = _run_diloco(device, factory, 3, [True, False, False, True, True], True)
+    assert m.current_step() == 3
+    m.shutdown(wait=False)
+
+
 def test_diloco_generic_manager_contract(device):
     """A foreign Manager (mock): per-parameter allreduce calls, kernels for the rest."""
     flag = [True]
@@ -385,6 +406,17 @@ def test_diloco_generic_manager_contract(device):
             assert_bits_equal(p.data, w)
         for p, w in zip(model.parameters(), want["momentum"]):
             assert_bits_equal(outer.state[p]["momentum_buffer"], w)
+        # a sync that is not committed: the local changes are discarded, nothing else moves
+        flag[0] = False
+        with torch.no_grad():
+            for p in model.parameters():
+                p.data.add_(3e-3)
+                p.grad = torch.zeros_like(p)
+        inner.step()
+        for p, b, w, m in zip(model.parameters(), diloco._backup_parameters.values(), want["backup"], want["momentum"]):
+            assert_bits_equal(b, w)
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(outer.state[p]["momentum_buffer"], m)
 
 
 def test_diloco_gpt2_small_four_replicas(device):
@@ -801,6 +833,17 @@ def test_diloco_bucketized_on_gpu(device):
             assert_bits_equal(outer.state[p]["momentum_buffer"], m)
         for b, w in zip(diloco._backup_parameters.values(), want["backup"]):
             assert_bits_equal(b, w)
+        # a sync that is not committed: the local changes are discarded, nothing else moves
+        manager._client.should_commit = lambda *a, **k: False
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(2e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        inner.step()
+        for p, b, w, m in zip(model.parameters(), diloco._backup_parameters.values(), want["backup"], want["momentum"]):
+            assert_bits_equal(b, w)
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(outer.state[p]["momentum_buffer"], m)
     manager.shutdown(wait=False)
 
 

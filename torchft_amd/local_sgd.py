@@ -714,17 +714,25 @@ class DiLoCo(LocalSGD):
 
         bucketized = not fused and _is_native_manager(self._manager)
         grads = self._flat_like("grads", params)[1] if bucketized else self._grad_buffers(params)
+        # The reference restores the parameters before the vote (torchft/local_sgd.py:219) because
+        # its optimizer then steps on them.  The fused outer SGD computes the new parameters from
+        # the backup and the averaged pseudo-gradient and overwrites the parameters without
+        # reading them, so on a committed step the restore would be written for nothing (one
+        # model-sized stream): with a fusable optimizer it is done only when the step is NOT
+        # committed.  Any other optimizer gets its restore first, as in the reference.
+        restore_first = plan is None
+        restored = False
         if fused:
-            # pseudo-gradient, replica sum, divide and restore: one launch
+            # pseudo-gradient, replica sum and divide (and the restore, if it comes first): one launch
             for p, g in zip(live, grads):
                 p.grad = g
-            self._manager.pseudograd_allreduce(grads, params, backups, restore_params=True).wait()
-            if self._manager.errored() is not None:
-                self._restore_parameters()  # the launch that restores did not happen
+            self._manager.pseudograd_allreduce(grads, params, backups, restore_params=restore_first).wait()
+            restored = restore_first and self._manager.errored() is None
         elif bucketized:
-            # pseudo-gradients written straight into one flat buffer (and the parameters
-            # restored) by one launch, then ONE collective for the whole model
-            self._local_pseudograd(grads, params, backups, restore_params=True)
+            # pseudo-gradients written straight into one flat buffer by one launch, then ONE
+            # collective for the whole model
+            self._local_pseudograd(grads, params, backups, restore_params=restore_first)
+            restored = restore_first
             for p, g in zip(live, grads):
                 p.grad = g
             works = [self._manager.allreduce(flat) for flat in self._flat_like("grads", params)[0].values()]
@@ -736,10 +744,14 @@ class DiLoCo(LocalSGD):
             for p, g in zip(live, grads):
                 p.grad = g
             self._average_grads()
+        if restore_first and not restored:
             self._restore_parameters()
+            restored = True
 
         if self._manager.should_commit():
             self._outer_step(params, backups, grads, plan)
+        elif not restored:
+            self._restore_parameters()
         self._outer_optimizer.zero_grad()
 
     def _local_pseudograd(
