@@ -760,8 +760,6 @@ def bench_host_backup(args) -> Dict[str, object]:
     n_params = sum(t.numel() for t in params)
     nbytes = 4 * n_params
     backup = _PackedHostBackup([(str(i), t) for i, t in enumerate(params)], pin_memory=True)
-    stream = torch.cuda.current_stream(dev)
-
     def ev():
         return torch.cuda.Event(enable_timing=True)
 

@@ -1267,7 +1267,7 @@ def test_diloco_keeps_its_prepared_sync_and_notices_every_change(cpu_ops):
         bound = diloco._bound
 
         # the outer optimizer's state is replaced (load_state_dict after healing)
-        saved = copy_state = outer.state_dict()
+        copy_state = outer.state_dict()
         outer.load_state_dict(copy_state)
         state["bufs"] = [outer.state[p]["momentum_buffer"].clone() for p in model.parameters()]
         plan = diloco._plan

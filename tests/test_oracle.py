@@ -5,7 +5,6 @@ the reference's tests, torch library routines (torch.optim.SGD, the DDP Reducer'
 assignment, torch.save/torch.load), closed forms, float64 brute force and invariants.
 """
 
-import numpy as np
 import pytest
 import torch
 import torch.distributed as dist

@@ -15,7 +15,6 @@ import time
 from datetime import timedelta
 from typing import Callable, List, Optional, Tuple, TypeVar
 
-import torch
 from torch.futures import Future
 
 T = TypeVar("T")
