@@ -966,6 +966,42 @@ def test_diloco_bucketized_one_collective_per_sync(cpu_ops):
     manager.shutdown(wait=False)
 
 
+@pytest.mark.parametrize("outer_kind", ["sgd", "adam"])
+def test_diloco_bucketized_failed_collective_discards_the_step(cpu_ops, outer_kind):
+    """The collective fails: the error is latched, the vote is no, and the parameters go back to
+    the backup whether the restore was part of the first launch (an optimizer that steps on
+    the parameters) or left for the no-commit branch (the fused SGD)."""
+    torch.manual_seed(0)
+    model = SimpleModel()
+
+    class Failing(_DoublingPG):
+        def allreduce(self, tensors, opts):
+            self.calls.append([t.numel() for t in tensors])
+            raise RuntimeError("injected collective failure")
+
+    pg = Failing()
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = (optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True) if outer_kind == "sgd"
+             else optim.Adam(model.parameters(), lr=1e-3))
+    backup = [p.data.clone() for p in model.parameters()]
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1e-3 * torch.randn_like(p))
+                p.grad = torch.zeros_like(p)
+        inner.step()
+        assert len(pg.calls) == 1 and manager.errored() is not None
+        for p, b, w in zip(model.parameters(), diloco._backup_parameters.values(), backup):
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(b, w)
+        assert outer.state_dict()["state"] == {}
+        assert all(p.grad is None for p in model.parameters())
+        assert "mt_outer_sgd" not in cpu_ops.calls
+    manager.shutdown(wait=False)
+
+
 def test_local_sgd_bucketized_one_collective_per_sync(cpu_ops):
     torch.manual_seed(0)
     model = SimpleModel()
