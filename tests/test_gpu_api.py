@@ -270,7 +270,7 @@ def test_localsgd_mlp_two_replicas(device):
     manager.shutdown(wait=False)
 
 
-def _run_diloco(device, manager_factory, n_replicas, commits, fused_expected):
+def _run_diloco(device, manager_factory, n_replicas, commits, fused_expected, backup_device=None, mutate_host_backup=False):
     torch.manual_seed(0)
     model = Tiny().to(device)
     peers, lookup = peer_world(model, n_replicas)
@@ -280,7 +280,7 @@ def _run_diloco(device, manager_factory, n_replicas, commits, fused_expected):
     backup = cpu(p.data for p in model.parameters())
     bufs = None
     gen = torch.Generator().manual_seed(9)
-    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+    with DiLoCo(manager, model, inner, outer, sync_every=1, backup_device=backup_device) as diloco:
         for step, commit in enumerate(commits):
             commit_flag[0] = commit
             for k, peer in enumerate(peers):
@@ -297,7 +297,18 @@ def _run_diloco(device, manager_factory, n_replicas, commits, fused_expected):
             want = O.diloco_perform_sync(
                 [local] + [cpu(q.data for q in peer.parameters()) for peer in peers], backup, bufs,
                 [True] * n_replicas, n_replicas, commit, lr=0.7, momentum=0.9, nesterov=True)
+            if mutate_host_backup and step == 2:
+                # the backup tensors are the user's to write between syncs: the next sync reads them
+                diloco._host_backup.wait()
+                for b, old_b in zip(diloco._backup_parameters.values(), backup):
+                    b.mul_(1.0009765625)
+                    old_b.mul_(1.0009765625)
+                want = O.diloco_perform_sync(
+                    [local] + [cpu(q.data for q in peer.parameters()) for peer in peers], backup, bufs,
+                    [True] * n_replicas, n_replicas, commit, lr=0.7, momentum=0.9, nesterov=True)
             inner.step()  # zero gradient: parameters unchanged, post hook runs the sync
+            if diloco._host_backup is not None:
+                diloco._host_backup.wait()  # the refreshed backup crosses PCIe on a side stream
             for p, w in zip(model.parameters(), want["params"]):
                 assert_bits_equal(p.data, w, f"step {step} params")
             for (name, b), w in zip(diloco._backup_parameters.items(), want["backup"]):
@@ -348,6 +359,107 @@ def test_diloco_two_launches_when_the_reduction_may_fail_late(device):
     m = _run_diloco(device, factory, 3, [True, False, False, True, True], True)
     assert m.current_step() == 3
     m.shutdown(wait=False)
+
+
+@pytest.mark.parametrize("fails_only_at_launch", [True, False])
+def test_diloco_with_the_backup_in_host_memory(device, fails_only_at_launch):
+    """``backup_device="cpu"`` (torchft/local_sgd.py:185-203 takes it; :214 moves the backup to
+    the parameter's device per tensor): the kernels work on the backup's device-side staging
+    buffer, loaded from the pinned host buffer before every sync and sent back after a
+    committed one.  Single launch and two launches, committed and not, and a backup the user
+    has written between two syncs."""
+    flag = [True]
+
+    def factory(lookup):
+        pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+        pg.fails_only_at_launch = fails_only_at_launch
+
+        class Vote(StaticQuorum):
+            def should_commit(self, rank, step, should_commit, timeout):
+                return should_commit and flag[0]
+
+        return Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1, use_async_quorum=False, quorum_client=Vote(0, 2)), flag
+
+    m = _run_diloco(device, factory, 2, [True, False, True, True], True,
+                    backup_device=torch.device("cpu"), mutate_host_backup=True)
+    assert m.current_step() == 3
+    m.shutdown(wait=False)
+
+
+def test_diloco_with_backup_tensors_the_user_put_in_place(device):
+    """``_backup_parameters`` replaced by plain host tensors (a load_state_dict after healing,
+    torchft/manager_integ_test.py:279): every sync reads them and a committed one rewrites them."""
+    torch.manual_seed(0)
+    model = Tiny().to(device)
+    peers, lookup = peer_world(model, 2)
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    gen = torch.Generator().manual_seed(5)
+    with DiLoCo(manager, model, inner, outer, sync_every=1) as diloco:
+        mine = {n: (b.cpu() + 1e-3 * torch.randn(b.shape, generator=gen)) for n, b in diloco._backup_parameters.items()}
+        diloco._backup_parameters = mine
+        backup, bufs = [b.clone() for b in mine.values()], None
+        for step in range(3):
+            for q, b in zip(peers[0].parameters(), backup):
+                q.data.copy_((b + 1e-3 * torch.randn(b.shape, generator=gen)).to(device))
+            with torch.no_grad():
+                for p, b in zip(model.parameters(), backup):
+                    p.data.copy_((b + 2e-3 * torch.randn(b.shape, generator=gen)).to(device))
+                    p.grad = torch.zeros_like(p)
+            local = cpu(p.data for p in model.parameters())
+            want = O.diloco_perform_sync([local, cpu(q.data for q in peers[0].parameters())], backup, bufs,
+                                         [True, True], 2, True, lr=0.7, momentum=0.9, nesterov=True)
+            inner.step()
+            assert diloco._backup_parameters is mine
+            for p, b, w, wb, wm in zip(model.parameters(), mine.values(), want["params"], want["backup"], want["momentum"]):
+                assert b.device.type == "cpu"
+                assert_bits_equal(p.data, w, f"step {step} params")
+                assert_bits_equal(b, wb, f"step {step} backup")
+                assert_bits_equal(outer.state[p]["momentum_buffer"], wm, f"step {step} momentum")
+            backup, bufs = want["backup"], want["momentum"]
+    manager.shutdown(wait=False)
+
+
+def test_localsgd_with_the_backup_in_host_memory_is_one_launch_and_one_transfer(device):
+    """Local replicas and a pinned host backup: the average goes to the parameters and to the
+    backup's staging buffer in one launch; the checker's bits, committed and not."""
+    torch.manual_seed(0)
+    model = MLP().to(device)
+    peers, lookup = peer_world(model, 2)
+    flag = [True]
+
+    class Vote(StaticQuorum):
+        def should_commit(self, rank, step, should_commit, timeout):
+            return should_commit and flag[0]
+
+    pg = ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=Vote(0, 2))
+    optimizer = optim.SGD(model.parameters(), lr=1e-3)
+    gen = torch.Generator().manual_seed(11)
+    with LocalSGD(manager, model, optimizer, sync_every=1, backup_device=torch.device("cpu")) as lsgd:
+        lsgd._host_backup.wait()
+        backup = [b.clone() for b in lsgd._backup_parameters.values()]
+        for step, commit in enumerate([True, False, True]):
+            flag[0] = commit
+            for q in peers[0].parameters():
+                q.data.add_((1e-3 * torch.randn(q.shape, generator=gen)).to(device))
+            with torch.no_grad():
+                for p in model.parameters():
+                    p.add_((1e-3 * torch.randn(p.shape, generator=gen)).to(device))
+                    p.grad = torch.zeros_like(p)
+            local = cpu(p.data for p in model.parameters())
+            want = O.localsgd_perform_sync([local, cpu(q.data for q in peers[0].parameters())], backup,
+                                           [True, True], 2, commit)
+            optimizer.step()
+            lsgd._host_backup.wait()
+            for p, b, w, wb in zip(model.parameters(), lsgd._backup_parameters.values(), want["params"], want["backup"]):
+                assert b.is_pinned()
+                assert_bits_equal(p.data, w, f"step {step} params")
+                assert_bits_equal(b, wb, f"step {step} backup")
+            backup = want["backup"]
+    manager.shutdown(wait=False)
 
 
 def test_diloco_generic_manager_contract(device):

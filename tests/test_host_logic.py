@@ -1358,6 +1358,58 @@ def test_peer_lookups_are_repeated_unless_declared_stable(cpu_ops):
     manager.shutdown(wait=False)
 
 
+def test_diloco_mirrors_a_backup_kept_elsewhere(cpu_ops, monkeypatch):
+    """Backup tensors that do not live with the parameters (host memory, a user's own tensors)
+    are copied into device buffers for the sync and written back after a committed step; a
+    step that is not committed leaves them alone and restores the parameters from them."""
+    from torchft_amd import local_sgd
+
+    torch.manual_seed(0)
+    model = SimpleModel()
+    peers, pg, _ = _stable_world(model, 2)
+    flag = [True]
+
+    class Vote(StaticQuorum):
+        def should_commit(self, rank, step, should_commit, timeout):
+            return should_commit and flag[0]
+
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=1,
+                      use_async_quorum=False, quorum_client=Vote(0, 2))
+    inner = optim.SGD(model.parameters(), lr=0.1)
+    outer = optim.SGD(model.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+    elsewhere = set()
+    monkeypatch.setattr(local_sgd.LocalSGD, "_on_device", staticmethod(
+        lambda params, backups: bool(params) and not any(b.data_ptr() in elsewhere for b in backups)))
+    monkeypatch.setattr(local_sgd.LocalSGD, "_on_one_gpu", staticmethod(lambda params: bool(params)))
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda device=None: MagicMock())
+    state = {"backup": [p.data.clone() for p in model.parameters()], "bufs": None}
+    with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9) as diloco:
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+        mine = {k: v.clone() for k, v in diloco._backup_parameters.items()}
+        elsewhere.update(v.data_ptr() for v in mine.values())
+        diloco._backup_parameters = mine
+        for _ in range(2):
+            _checked_diloco_sync(diloco, model, peers, outer, state)   # compares ``mine`` with the checker
+            assert diloco._backup_parameters is mine
+        mirror = diloco._flat["backup_mirror"][2]
+        assert all(m.data_ptr() != b.data_ptr() for m, b in zip(mirror, mine.values()))
+        # not committed: parameters back to the backup, backup and momentum untouched
+        flag[0] = False
+        before = [v.clone() for v in mine.values()]
+        momentum = [outer.state[p]["momentum_buffer"].clone() for p in model.parameters()]
+        with torch.no_grad():
+            for p in model.parameters():
+                p.add_(1e-3 * torch.randn_like(p))
+        diloco.sync()
+        for p, b, w, m in zip(model.parameters(), mine.values(), before, momentum):
+            assert_bits_equal(b, w)
+            assert_bits_equal(p.data, w)
+            assert_bits_equal(outer.state[p]["momentum_buffer"], m)
+        flag[0] = True
+        _checked_diloco_sync(diloco, model, peers, outer, state)
+    manager.shutdown(wait=False)
+
+
 def test_local_sgd_keeps_its_prepared_average(cpu_ops):
     torch.manual_seed(0)
     model = SimpleModel()

@@ -117,6 +117,11 @@ class _PackedHostBackup:
         self.staging_views = [
             self.staging[o : o + p.numel() * p.element_size()] for o, p in zip(offsets, params)
         ]
+        # the staging buffer seen as the parameters' device-side backup: the sync kernels read
+        # and write these, the staging buffer then crosses PCIe as it does after a save
+        self.device_views = [
+            v.view(p.dtype).view(p.shape) for v, p in zip(self.staging_views, params)
+        ]
         self.stream = torch.cuda.Stream(device=self.device)
         self.host_ready: Optional[torch.cuda.Event] = None  # the last save has reached the host
         self._tables: Dict[str, TensorTable] = {}
@@ -131,6 +136,19 @@ class _PackedHostBackup:
         if self.host_ready is not None:
             current.wait_event(self.host_ready)  # staging is free again
         self._tables["pack"] = ops.mt_copy(self.staging_views, params, table=self._tables.get("pack"))
+        self.publish()
+
+    def reserve(self) -> List[torch.Tensor]:
+        """``device_views`` for a kernel on the current stream to WRITE: waits (on the stream)
+        until the previous transfer has left the staging buffer."""
+        if self.host_ready is not None:
+            torch.cuda.current_stream(self.device).wait_event(self.host_ready)
+        return self.device_views
+
+    def publish(self) -> None:
+        """Sends the staging buffer, as the current stream leaves it, to the host on the side
+        stream (the tail of a save; also after a sync kernel has written ``device_views``)."""
+        current = torch.cuda.current_stream(self.device)
         packed = torch.cuda.Event()
         packed.record(current)
         self.stream.wait_event(packed)
@@ -138,6 +156,16 @@ class _PackedHostBackup:
             self.host.copy_(self.staging, non_blocking=True)
             self.host_ready = torch.cuda.Event()
             self.host_ready.record(self.stream)
+
+    def load(self) -> List[torch.Tensor]:
+        """Brings the host backup into the staging buffer (one transfer on the current stream)
+        and returns it as ``device_views``: the backup as the kernels read it.  The host
+        tensors are the user's to change between syncs, so this is done for every sync that
+        reads the backup (the reference moves every tensor with ``.to(p.device)`` instead,
+        torchft/local_sgd.py:214)."""
+        self.wait()
+        self.staging.copy_(self.host, non_blocking=True)
+        return self.device_views
 
     def wait(self) -> None:
         """Blocks until the host copy is complete (before anything reads the backup)."""
@@ -364,20 +392,38 @@ class LocalSGD:
         self._local_step = 0
 
     def _fused(self, params: Sequence[torch.Tensor], backups: Sequence[torch.Tensor]) -> bool:
-        bound = self._bound
-        on_device = (
-            bound.on_device if bound is not None and bound.params is params
-            else self._on_device(params, backups)
-        )
         return (
-            on_device
+            self._together(params, backups)
             and _is_native_manager(self._manager)
             and self._manager.supports_fused_sync()
         )
 
+    def _together(self, params: Sequence[torch.Tensor], backups: Sequence[torch.Tensor]) -> bool:
+        """``_on_device``, remembered for the bound lists."""
+        bound = self._bound
+        if bound is not None and bound.params is params and bound.backups is backups:
+            return bound.on_device
+        return self._on_device(params, backups)
+
+    @staticmethod
+    def _on_one_gpu(params: Sequence[torch.Tensor]) -> bool:
+        return bool(params) and all(p.is_cuda and p.device == params[0].device for p in params)
+
     def _perform_sync(self) -> None:
         """Average, then keep the result (commit) or roll back (torchft/local_sgd.py:151-162)."""
         _, params, backups = self._named()
+        hb = self._host_backup
+        if (
+            hb is not None
+            and hb.owns(backups)
+            and self._manager.reduction_fails_only_at_launch()
+            and self._fused(params, hb.device_views)
+        ):
+            # backup in pinned host memory: the launch writes the average to the parameters and
+            # to the backup's device-side staging buffer, which then crosses PCIe once
+            if self._average_single_launch(params, hb.reserve()):
+                hb.publish()
+            return
         if self._fused(params, backups):
             if self._manager.reduction_fails_only_at_launch():
                 self._average_single_launch(params, backups)
@@ -392,7 +438,7 @@ class LocalSGD:
         else:
             self._restore_parameters()
 
-    def _average_single_launch(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> None:
+    def _average_single_launch(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> bool:
         """A local reduction cannot fail once launched, so the commit decision is taken
         first and the sync is ONE launch: the average written to the parameters and the
         backup together, or (no commit) a plain restore.  Everything that can fail for a
@@ -403,7 +449,7 @@ class LocalSGD:
 
         The prepared launches are kept: as long as the parameters, the backups and the
         peers' buffers are the ones of the previous sync, nothing is rebuilt or compared
-        tensor by tensor."""
+        tensor by tensor.  Returns whether the step was committed (``backups`` written)."""
         manager = self._manager
         manager.wait_quorum()  # should_commit reads the quorum's results (async quorum)
         launches = []
@@ -435,8 +481,9 @@ class LocalSGD:
                 self._tables[key] = ops.mt_reduce_avg(
                     outs, reps, mask, manager.num_participants(), table=table, table_is_current=True
                 )
-        else:
-            self._restore_parameters()
+            return True
+        self._restore_parameters()
+        return False
 
     def _average_bucketized(self, params: List[torch.Tensor]) -> None:
         """Flatten (one launch), ONE ``manager.allreduce`` per dtype, unflatten (one launch)."""
@@ -696,21 +743,47 @@ class DiLoCo(LocalSGD):
         """Pseudo-gradients, their average over the replicas, restore, and (on commit)
         the outer step plus backup refresh (torchft/local_sgd.py:205-225)."""
         _, params, backups = self._named()
-        bound = self._bound
-        if not (bound.on_device if bound is not None and bound.params is params
-                else self._on_device(params, backups)):
+        if self._together(params, backups):
+            self._sync_with(params, backups)
+            return
+        if not self._on_one_gpu(params):
             raise RuntimeError(
-                "DiLoCo needs parameters and backup on one GPU (the kernels have no CPU path); "
-                "construct it with backup_device=None or the parameters' device"
+                "DiLoCo needs its parameters on one GPU (the kernels have no CPU path)"
             )
+        # The backup is kept elsewhere: in host memory (``backup_device="cpu"``) or in tensors
+        # the user has put in place.  The reference moves every backup tensor to the
+        # parameter's device for the subtraction (torchft/local_sgd.py:214); here the backup
+        # is brought into device buffers once per sync, the kernels work on those, and after a
+        # committed step they are written back.
+        hb = self._host_backup
+        packed = hb is not None and hb.owns(backups)
+        if packed:
+            mirror = hb.load()
+        else:
+            mirror = self._flat_like("backup_mirror", params)[1]
+            for m, b in zip(mirror, backups):
+                m.copy_(b, non_blocking=True)
+        if self._sync_with(params, mirror):
+            if packed:
+                hb.publish()
+            else:
+                for b, m in zip(backups, mirror):
+                    b.copy_(m, non_blocking=True)
+                if any(not b.is_cuda for b in backups):
+                    torch.cuda.current_stream(params[0].device).synchronize()
+
+    def _sync_with(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> bool:
+        """One sync over device-resident ``backups``.  Returns whether the kernels have
+        rewritten them (a committed step with a fusable outer SGD); any other outer optimizer
+        refreshes ``_backup_parameters`` itself through ``_save_parameters``."""
         live = self._param_objs
         plan = self._sgd_plan(params)
         fused = self._fused(params, backups)
 
         if fused and plan is not None and self._manager.reduction_fails_only_at_launch():
-            self._sync_single_launch(params, backups, plan)
+            committed = self._sync_single_launch(params, backups, plan)
             self._outer_optimizer.zero_grad()
-            return
+            return committed
 
         bucketized = not fused and _is_native_manager(self._manager)
         grads = self._flat_like("grads", params)[1] if bucketized else self._grad_buffers(params)
@@ -745,14 +818,25 @@ class DiLoCo(LocalSGD):
                 p.grad = g
             self._average_grads()
         if restore_first and not restored:
-            self._restore_parameters()
+            self._restore_from(params, backups)
             restored = True
 
-        if self._manager.should_commit():
+        committed = self._manager.should_commit()
+        if committed:
             self._outer_step(params, backups, grads, plan)
         elif not restored:
-            self._restore_parameters()
+            self._restore_from(params, backups)
         self._outer_optimizer.zero_grad()
+        return committed and plan is not None
+
+    def _restore_from(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> None:
+        """``_restore_parameters`` from the device-resident form of the backup this sync works
+        on (the bound backup itself, or its mirror)."""
+        bound = self._bound
+        if bound is not None and bound.backups is backups:
+            self._restore_parameters()
+        else:
+            self._copy("restore_mirror", params, backups, blocking=True)
 
     def _local_pseudograd(
         self,
@@ -776,12 +860,13 @@ class DiLoCo(LocalSGD):
         params: List[torch.Tensor],
         backups: List[torch.Tensor],
         plan: List[Tuple[List[int], ops.OuterSGD, bool]],
-    ) -> None:
+    ) -> bool:
         """The reduction is local and cannot fail once launched, so the commit decision
         can be taken first and the whole sync becomes one launch per parameter group:
         either the fully fused step, or (no commit) a plain restore.  The prepared launches
         (tensor lists and their validated table) are kept for as long as the parameters,
-        the backups, the plan and the peers' buffers are those of the previous sync."""
+        the backups, the plan and the peers' buffers are those of the previous sync.  Returns
+        whether the step was committed."""
         manager = self._manager
         manager.wait_quorum()
         launches = []
@@ -830,8 +915,9 @@ class DiLoCo(LocalSGD):
                 )
                 if first and cols["bufs"] is not None:
                     self._attach_momentum(idx, cols["bufs"])
-        else:
-            self._restore_parameters()
+            return True
+        self._restore_from(params, backups)
+        return False
 
     def _average_grads(self) -> None:
         """One ``manager.allreduce`` per pseudo-gradient (torchft/local_sgd.py:227-239)."""
