@@ -39,6 +39,7 @@ def cpu_ops(monkeypatch):
     monkeypatch.setattr(
         local_sgd.LocalSGD, "_on_device", staticmethod(lambda params, backups: bool(params))
     )
+    monkeypatch.setattr(local_sgd.LocalSGD, "_on_one_gpu", staticmethod(lambda params: bool(params)))
     fake_backend.calls.clear()
     return fake_backend
 

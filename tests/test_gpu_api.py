@@ -959,7 +959,8 @@ def test_diloco_bucketized_on_gpu(device):
     manager.shutdown(wait=False)
 
 
-def test_local_sgd_bucketized_on_gpu(device):
+@pytest.mark.parametrize("backup_device", [None, torch.device("cpu")])
+def test_local_sgd_bucketized_on_gpu(device, backup_device):
     torch.manual_seed(0)
     model = MLP().to(device)
     peer_params = [p.data.cpu() + 1e-3 * torch.randn(p.shape) for p in model.parameters()]
@@ -967,7 +968,9 @@ def test_local_sgd_bucketized_on_gpu(device):
     pg = _PlainLocalPG(lambda t: peer_flat)
     manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False, quorum_client=StaticQuorum(0, 2))
     optimizer = optim.SGD(model.parameters(), lr=0.1)
-    with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
+    with LocalSGD(manager, model, optimizer, sync_every=1, backup_device=backup_device) as lsgd:
+        if lsgd._host_backup is not None:
+            lsgd._host_backup.wait()
         backup = cpu(lsgd._backup_parameters.values())
         with torch.no_grad():
             for p in model.parameters():
@@ -976,7 +979,9 @@ def test_local_sgd_bucketized_on_gpu(device):
         local = cpu(p.data for p in model.parameters())
         want = O.localsgd_perform_sync([local, peer_params], backup, [True, True], 2, True)
         optimizer.step()
-        assert pg.calls == [sum(b.numel() for b in backup)]
+        if lsgd._host_backup is not None:
+            lsgd._host_backup.wait()
+        assert pg.calls == [sum(b.numel() for b in backup)]  # one collective wherever the backup is kept
         for p, w in zip(model.parameters(), want["params"]):
             assert_bits_equal(p.data, w)
         for b, w in zip(lsgd._backup_parameters.values(), want["backup"]):

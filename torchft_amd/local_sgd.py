@@ -416,8 +416,8 @@ class LocalSGD:
         if (
             hb is not None
             and hb.owns(backups)
-            and self._manager.reduction_fails_only_at_launch()
             and self._fused(params, hb.device_views)
+            and self._manager.reduction_fails_only_at_launch()
         ):
             # backup in pinned host memory: the launch writes the average to the parameters and
             # to the backup's device-side staging buffer, which then crosses PCIe once
@@ -429,8 +429,8 @@ class LocalSGD:
                 self._average_single_launch(params, backups)
                 return
             self._manager.allreduce_tensors(params).wait()
-        elif _is_native_manager(self._manager) and self._on_device(params, backups):
-            self._average_bucketized(params)
+        elif _is_native_manager(self._manager) and self._on_one_gpu(params):
+            self._average_bucketized(params)  # wherever the backup is kept
         else:
             self._average()
         if self._manager.should_commit():
