@@ -831,7 +831,61 @@ def bench_host_backup(args) -> Dict[str, object]:
         "compute_launch_during_transfer_ms": mean(overlapped),
         "per_tensor_copies_on_training_stream_ms": mean(per_tensor),
     }
+    del backup, out_t
+    torch.cuda.empty_cache()
+    out["diloco_sync_with_host_backup"] = diloco_sync_with_host_backup(params, other, n_params)
     return out
+
+
+def diloco_sync_with_host_backup(params: List[torch.Tensor], peer: List[torch.Tensor], n_params: int) -> Dict[str, object]:
+    """``DiLoCo(..., backup_device="cpu").sync()`` on the same tensors: the backup comes from
+    pinned host memory before the launch and goes back after it (the reference moves every
+    backup tensor with ``.to(p.device)`` inside the sync, torchft/local_sgd.py:214)."""
+    from torch import nn
+
+    from torchft_amd import DiLoCo, Manager, ProcessGroupLocalReplicas, StaticQuorum
+
+    class Bag(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList([nn.Parameter(t) for t in params])
+
+    model = Bag()
+    index = {p.data_ptr(): i for i, p in enumerate(model.parameters())}
+    pg = ProcessGroupLocalReplicas(0, 2, peer_lookup=lambda t: [peer[index[t.data_ptr()]]], peers_are_stable=True)
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = torch.optim.SGD(model.parameters(), lr=0.1)
+    outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
+    stream_ms, host_ms = [], []
+    with DiLoCo(manager, model, inner, outer, sync_every=10 ** 9, backup_device=torch.device("cpu")) as diloco:
+        diloco.sync()  # creates the momentum
+        for it in range(2 + 4):
+            diloco._host_backup.wait()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            a.record()
+            diloco.sync()
+            b.record()
+            b.synchronize()
+            diloco._host_backup.wait()
+            if it >= 2:
+                stream_ms.append(a.elapsed_time(b))
+                host_ms.append((time.perf_counter() - t0) * 1e3)
+        for i in (0, len(params) - 1):
+            if not torch.equal(list(diloco._backup_parameters.values())[i], params[i].cpu()):
+                raise RuntimeError("output check failed: host backup != parameters after a committed sync")
+    manager.shutdown(wait=False)
+    mean = lambda xs: sum(xs) / len(xs)
+    nbytes = 4 * n_params
+    return {
+        "training_stream_held_ms": mean(stream_ms),
+        "backup_on_host_again_after_ms": mean(host_ms),
+        "GB": nbytes / 1e9,
+        "note": "stream held = one host-to-device transfer of the backup + the fused launch; the "
+                "transfer back overlaps what the stream does next",
+    }
 
 
 def bench_ddp_buckets(args, form: str = "hook_order") -> Dict[str, object]:
