@@ -237,6 +237,22 @@ def test_localsgd_on_fp64_parameters(device):
 # LocalSGD / DiLoCo
 # ---------------------------------------------------------------------------
 
+def test_wrappers_refuse_what_the_kernels_cannot_stream(device):
+    """A configuration error is raised where the wrapper is constructed, not latched as a failed
+    all-reduce on every sync: integer parameters, and parameters that are strided views."""
+    manager = create_autospec(Manager)
+    manager._use_async_quorum = False
+    model = nn.Linear(8, 8).to(device)
+    model.weight = nn.Parameter(model.weight.data.t())  # a transposed view: not contiguous
+    with pytest.raises(ValueError, match="not contiguous"):
+        LocalSGD(manager, model, optim.SGD(model.parameters(), lr=0.1), sync_every=2)
+    model = nn.Linear(8, 8).to(device)
+    model.half()
+    model.weight = nn.Parameter(model.weight.data.to(torch.float64))
+    with pytest.raises(TypeError, match="float64"):
+        DiLoCo(manager, model, optim.SGD(model.parameters(), lr=0.1), optim.SGD(model.parameters(), lr=0.7), sync_every=2)
+
+
 def test_localsgd_mlp_two_replicas(device):
     """The CPU-runnable configuration: 3-layer MLP, 2 replicas = backup + N(0, 1e-3),
     sync_every=1, result written into the parameters; the average is done on the GPU."""

@@ -263,6 +263,13 @@ class LocalSGD:
                     f"{type(self).__name__}: GPU parameters of {', '.join(bad)}; its kernels take "
                     + ", ".join(str(d).replace("torch.", "") for d in self._DTYPES)
                 )
+            strided = [name for name, p in named if p.is_cuda and not p.is_contiguous()]
+            if strided:
+                raise ValueError(
+                    f"{type(self).__name__}: parameters that are not contiguous in memory "
+                    f"({', '.join(strided[:4])}{', ...' if len(strided) > 4 else ''}): the kernels "
+                    "stream whole tensors; make them contiguous before wrapping the model"
+                )
         # the first sync needs a valid backup
         self._save_parameters()
 
