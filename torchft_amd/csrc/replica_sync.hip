@@ -751,7 +751,8 @@ enum Family { kFamReduce, kFamDiloco, kFamPseudograd, kFamOuterSgd, kFamCopy };
 // the Llama-3-8B and GPT-2-small workloads.  `traffic` is the launch's algorithmic bytes.
 // Launches that move less than a few GB finish in under a millisecond and are dominated by
 // the ramp and tail of the in-flight window: short runs and 5 resident workgroups per CU
-// (32 KiB of unused LDS each) are worth 5-10 % there.  Large launches still gain 1-5 % from
+// (32 KiB of unused LDS each; 3 of 48 KiB for the fused step, whose workgroups hold seven
+// to eleven streams in flight) are worth 5-10 % there.  Large launches still gain 1-5 % from
 // runs of 128-256 slabs with 2-3 resident workgroups per CU; the plain copy is best left
 // alone.
 Shape pick_shape(Family fam, uint64_t traffic) {
@@ -761,7 +762,7 @@ Shape pick_shape(Family fam, uint64_t traffic) {
   if (small) {
     s.unroll = fam == kFamDiloco ? 1 : 2;
     s.run_log2 = fam == kFamDiloco ? 7 : 6;
-    s.lds_bytes = 32u << 10;
+    s.lds_bytes = (fam == kFamDiloco ? 48u : 32u) << 10;
   } else if (fam == kFamDiloco || fam == kFamOuterSgd) {
     s.run_log2 = 8;
     s.lds_bytes = 64u << 10;

@@ -493,8 +493,8 @@ def allocate_apart(
     like: Sequence[torch.Tensor], n_copies: int
 ) -> Optional[List[List[torch.Tensor]]]:
     """``n_copies`` (1 to 3) sets of uninitialised tensors shaped like ``like``, every tensor
-    of every copy in a bank group other than its model tensor's: the group after it in
-    order of discovery; what does not fit there goes to the remaining group, and only then
+    of every copy in a bank group other than its model tensor's: the first one found that is
+    not the tensor's own; what does not fit there goes to the remaining group, and only then
     to the tensor's own.  Returns None when placement does not apply (switched off, not on
     a GPU, model too small, no group structure found); the caller then allocates as it
     always did."""
@@ -551,11 +551,13 @@ def _allocate_apart(
             pool.blocks = []
         pool.release_unused()
         return None
-    n_known = len(pool.map.anchors)
     groups = groups_of_tensors(pool, like)
-    # a tensor in none of the known groups lies in the one not reached yet: every known group
-    # is "another group" for it; the first is as good as any
-    wanted = [((0 if g is None else g + 1) % n_known) for g in groups]
+    # The group the copies of a tensor should go to: the first known group that is not the
+    # tensor's own (for a tensor in none of the known groups, which lies in the one not reached
+    # yet, every known group is "another group").  The choice does not depend on how many groups
+    # are known, so a later search, which may know one more, still prefers the blocks an
+    # earlier one has classified.
+    wanted = [(1 if g == 0 else 0) for g in groups]
     order = sorted(range(len(like)), key=lambda i: -sizes[i])  # large tensors first: they pack better
     need: Dict[int, int] = {}
     for size, w in zip(sizes, wanted):
