@@ -1414,11 +1414,21 @@ def api_child_main(args) -> int:
 def run_api_child(child) -> object:
     """Gives the child its go-ahead and returns the api sub-record, or None if it failed."""
     try:
+        import queue
+        import threading
+
         child.stdin.write("go\n")
         child.stdin.flush()
-        line = child.stdout.readline()
-        while line and not line.startswith("{"):
+        lines: "queue.Queue[str]" = queue.Queue()
+
+        def read_record() -> None:
             line = child.stdout.readline()
+            while line and not line.startswith("{"):
+                line = child.stdout.readline()
+            lines.put(line)
+
+        threading.Thread(target=read_record, daemon=True).start()
+        line = lines.get(timeout=600)  # a child that hangs must not hang the headline line
         child.wait(timeout=60)
         record = api_record(json.loads(line))
         record["process"] = ("a process of its own, started before the headline run touched the GPU and "
