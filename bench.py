@@ -475,6 +475,8 @@ def bench_diloco_api(args, which: str = "llama3_8b") -> Dict[str, object]:
             n_syncs += 10
         bufs = [outer.state[p]["momentum_buffer"] for p in model.parameters()]
         checked = replay.check(n_syncs, [p.data for p in model.parameters()], backups, bufs, dtype)
+        where = stream_groups(dev, {"p": [p.data for p in model.parameters()], "x1": peers[0],
+                                    "b": backups, "buf": bufs})
     manager.shutdown(wait=False)
     metric = HEADLINE_METRIC if which == "llama3_8b" else "outer-sync params/sec, GPT-2-small DiLoCo"
     out = base_line(args, metric + " (through DiLoCo.sync())", n_params / (wall_ms * 1e-3),
@@ -489,11 +491,33 @@ def bench_diloco_api(args, which: str = "llama3_8b") -> Dict[str, object]:
     out["roofline"] = roofline(n_params * (n_rep + 5) * esize, kernel_ms,
                                f"mt_stream_kernel<{'F32' if esize == 4 else 'BF16'}, DilocoFusedOp<{n_rep}>>")
     out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
+    if where:
+        out["config"]["hbm_bank_groups"] = where
     timed = host_ms[args.warmup:]
     out["host_ms_per_sync"] = sum(timed) / len(timed)
     if isolated_ms:
         out["isolated_sync_ms"] = sum(isolated_ms) / len(isolated_ms)
     return out
+
+
+def stream_groups(dev: torch.device, streams: Dict[str, List[torch.Tensor]], samples: int = 8) -> str:
+    """Which HBM bank group (A, B, C in order of discovery; ? = none of the known ones) a
+    few large tensors of every stream lie in, found with the library's own probe against the
+    reference buffers its placement search has kept; empty if there was no search."""
+    from torchft_amd import hbm_placement
+
+    state = hbm_placement.device_state(dev)
+    if len(state.map.anchors) < 2:
+        return ""
+    first = next(iter(streams.values()))
+    big = [i for i, t in enumerate(first) if t.numel() * t.element_size() >= hbm_placement.MIN_PROBE_BYTES]
+    if not big:
+        return ""
+    pick = big[:: max(1, len(big) // samples)][:samples]
+    with state.lock:
+        return " ".join(
+            name + ":" + "".join("?" if g is None else "ABC"[g] for g in (state.map.group_of(ts[i]) for i in pick))
+            for name, ts in streams.items())
 
 
 def api_record(line: Dict[str, object]) -> Dict[str, object]:
@@ -510,6 +534,7 @@ def api_record(line: Dict[str, object]) -> Dict[str, object]:
         "frac": roof["frac"],
         "host_ms_per_sync": line["host_ms_per_sync"],
         "output_check": line["config"]["output_check"],
+        "hbm_bank_groups": line["config"].get("hbm_bank_groups", ""),
     }
 
 

@@ -357,6 +357,32 @@ def test_a_model_of_many_tensors_is_classified_from_a_sample(small_constants, mo
     before = dev.probes
     groups = H.groups_of_tensors(pool, like)
     measured = (dev.probes - before) / len(pool.map.anchors)
-    assert measured <= 5 + 8, "a sample and one bisection, not one probe per tensor"
+    assert measured <= 5 + 8 + 8, "a sample, one bisection and the checks, not one probe per tensor"
     names = {truth[0]: groups[0], truth[-1]: groups[-1]}
     assert [names[g] for g in truth] == groups
+
+
+def test_a_model_scattered_over_the_groups_is_measured_tensor_by_tensor(small_constants, monkeypatch):
+    """Parameters allocated into memory that others had used and freed can alternate between
+    groups from one tensor to the next; a sample with bisection cannot see that, the checks
+    in between do, and then every probe-able tensor is measured."""
+    dev = FakeDevice(total=900 * MiB, group_bytes=100 * MiB)
+    flat = model_on(dev, [MiB // 2] * 80)            # 0-49 in group 0, 50-79 in group 1
+    like = [t for pair in zip(flat[:30], flat[50:80]) for t in pair] + flat[30:50]
+    truth = [dev.group_at(t) for t in like]
+    assert truth[:6] == [0, 1, 0, 1, 0, 1] and truth[-20:] == [0] * 20
+    pool = make_pool(dev, monkeypatch)
+    pool.grow_until(lambda pl: len(pl.map.anchors) >= 3)
+    before = dev.probes
+    groups = H.groups_of_tensors(pool, like)
+    names = {}
+    for t, g in zip(truth, groups):
+        assert names.setdefault(t, g) == g, "one name per true group"
+    assert len(set(names.values())) == 2
+    assert (dev.probes - before) / len(pool.map.anchors) >= len(like)  # everything was measured
+    # and the placement follows: every copy outside its own tensor's group
+    state = pool.state
+    copies = H._allocate_apart(like, [t.numel() * 4 for t in like], 1, torch.device("cpu"), pool=pool, state=state)
+    assert copies is not None
+    for t, c in zip(like, copies[0]):
+        assert dev.group_at(c) != dev.group_at(t)

@@ -83,6 +83,7 @@ RELATIVE_CONTRAST = 1.06     # own-group probe time / next longest, with all thr
 NO_STRUCTURE_BYTES = 110 << 30  # this much memory in ONE group: the device has no such groups
 MIN_MODEL_BYTES = 256 << 20  # smaller models are left alone (a GPT-2-small of 0.5 GB still gains 1-2 %)
 MODEL_SAMPLES = 5            # tensors of the model probed before any bisection
+MODEL_CHECKS = 8             # tensors in between measured afterwards, against what the sample predicts
 SEARCH_FRACTION = 0.75       # of the free device memory a search may hold, unless the environment says
 ALIGN = 256
 
@@ -425,52 +426,64 @@ class GroupedPool:
 
 def _sample_groups(pool: GroupedPool, tensors: Sequence[torch.Tensor], probeable: List[int],
                    out: List[Optional[int]]) -> None:
-    """Fills ``out`` for the probe-able tensors.  A model's tensors are allocated one after
-    the other, so they lie in at most a few runs of one group each: a handful of probes
+    """Fills ``out`` for the probe-able tensors.  A model's tensors are usually allocated one
+    after the other, so they lie in at most a few runs of one group each: a handful of probes
     spread over the list, then bisection between neighbours that disagree, instead of one
-    probe per tensor."""
+    probe per tensor.  A few more tensors in between are then measured against what that
+    predicts for them; if one of them lies elsewhere (a model allocated into memory that
+    others had used and freed can alternate between groups from tensor to tensor), every
+    probe-able tensor is measured."""
     known = pool.state.known  # by address, like the blocks: valid until memory goes back to the driver
+    measured: Dict[int, Optional[int]] = {}
 
-    def probe(k: int) -> Optional[int]:
-        i = probeable[k]
-        if out[i] is None:
-            t = tensors[i]
+    def measure(k: int) -> Optional[int]:
+        if k not in measured:
+            t = tensors[probeable[k]]
             key, nbytes = t.data_ptr(), _as_bytes(t).numel()
             cached = known.get(("tensor", key))
             n_anchors = len(pool.map.anchors)
             # "in none of the known groups" is an answer too, for as long as no group is added
             if cached is not None and cached[0] == nbytes and (cached[1] is not None or cached[2] == n_anchors):
-                out[i] = cached[1]
+                measured[k] = cached[1]
                 pool.cache_hits += 1
             else:
-                out[i] = pool.map.group_of(t)
-                if _as_bytes(t).numel() >= MIN_PROBE_BYTES:
-                    known[("tensor", key)] = (nbytes, out[i], n_anchors)
-            probed.add(k)
-        return out[i]
+                measured[k] = pool.map.group_of(t)
+                if nbytes >= MIN_PROBE_BYTES:
+                    known[("tensor", key)] = (nbytes, measured[k], n_anchors)
+        return measured[k]
 
-    probed: set = set()
+    def predicted(k: int, among: List[int]) -> Optional[int]:
+        """The group of the nearest measured tensor in list order."""
+        return measured[min(among, key=lambda j: (abs(j - k), j))]
+
     n = len(probeable)
     if n == 0:
         return
     picks = sorted({round(j * (n - 1) / max(MODEL_SAMPLES - 1, 1)) for j in range(MODEL_SAMPLES)})
     for k in picks:
-        probe(k)
+        measure(k)
     # bisect between sampled neighbours whose groups differ
     work = list(zip(picks, picks[1:]))
     while work:
         lo, hi = work.pop()
-        if hi - lo <= 1 or out[probeable[lo]] == out[probeable[hi]]:
+        if hi - lo <= 1 or measured[lo] == measured[hi]:
             continue
         mid = (lo + hi) // 2
-        probe(mid)
+        measure(mid)
         work += [(lo, mid), (mid, hi)]
-    # everything in between takes the group of the nearest probed tensor in list order
-    known = sorted(probed)
+    # does the picture of a few runs hold?  Tensors between the measured ones say
+    rest = [k for k in range(n) if k not in measured]
+    if rest:
+        basis = sorted(measured)
+        checks = sorted({rest[min(len(rest) - 1, int((j + 0.5) * len(rest) / MODEL_CHECKS))]
+                         for j in range(MODEL_CHECKS)})
+        expected = {k: predicted(k, basis) for k in checks}
+        if any(measure(k) != expected[k] for k in checks):
+            for k in rest:
+                measure(k)
+    basis = sorted(measured)
     for k in range(n):
-        if k not in probed:
-            nearest = min(known, key=lambda j: (abs(j - k), j))
-            out[probeable[k]] = out[probeable[nearest]]
+        out[probeable[k]] = measured[k] if k in measured else predicted(k, basis)
 
 
 def groups_of_tensors(pool: GroupedPool, tensors: Sequence[torch.Tensor]) -> List[Optional[int]]:
