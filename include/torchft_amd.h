@@ -60,7 +60,7 @@
 extern "C" {
 #endif
 
-#define TFT_ABI_VERSION 5
+#define TFT_ABI_VERSION 6
 #define TFT_MAX_REPLICAS 8 /* replica pointer columns per launch */
 #define TFT_MIN_CHUNK_ELEMS 8192u
 #define TFT_NOALLOC_MAX_TENSORS 4096u /* rows of the built-in table of the allocation-free entry */
@@ -171,6 +171,17 @@ int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
                           uint32_t participate_mask, uint32_t num_participants, int dtype,
                           int restore_p, void* stream);
 int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd, void* stream);
+
+/*
+ * Phase 2 when g still holds the SUM a collective has left in it: Manager.allreduce
+ * divides the summed buffer by num_participants in a pass of its own
+ * (torchft/manager.py:287); here the quotient is formed per element in registers,
+ *   g' = g / num_participants   (IEEE division; rounded to the storage type as the
+ *                                separate pass would have stored it),
+ * and the SGD update of tft_mt_outer_sgd runs on g'.  g itself is not written.
+ */
+int tft_mt_outer_sgd_of_sum(const tft_mt_table* table, uint32_t num_participants, int dtype,
+                            const tft_sgd_params* sgd, void* stream);
 
 /*
  * Allocation-free form of tft_mt_diloco_outer.  It has no counterpart in the

@@ -90,10 +90,14 @@ def _sgd_from_backup(t, params, backups, bufs, g32, sgd, first_step):
     backups[t].copy_(p)
 
 
-def mt_outer_sgd(params, backups, bufs, grads, sgd, first_step, table=None):
+def mt_outer_sgd(params, backups, bufs, grads, sgd, first_step, table=None, grads_are_sums_of=None):
     calls.append("mt_outer_sgd")
     for t in range(len(params)):
-        _sgd_from_backup(t, params, backups, bufs, grads[t].float(), sgd, first_step)
+        g32 = grads[t].float()
+        if grads_are_sums_of is not None:
+            # what Manager.allreduce's own division would have stored in the buffer
+            g32 = (g32 / float(grads_are_sums_of)).to(grads[t].dtype).float()
+        _sgd_from_backup(t, params, backups, bufs, g32, sgd, first_step)
     return FakeTable()
 
 

@@ -240,6 +240,70 @@ def test_diloco_two_phase_matches_fused_and_checker(device):
         assert_bits_equal(m[i], want["momentum"][i], f"momentum {name}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 7])
+def test_outer_sgd_of_a_sum_divides_like_the_pass_it_replaces(device, dtype, n):
+    """The gradient buffer holds the SUM a collective left in it.  Two ways to the same bits:
+    Manager.allreduce's own division over the buffer (``reduce_avg_`` with one replica and
+    ``num_participants = n``), then the outer SGD; or the outer SGD that divides on the way in.
+    Sums over the whole encoding of the storage type, ragged sizes, misaligned views."""
+    gen = torch.Generator().manual_seed(100 * n + int(dtype.itemsize))
+    sizes = [1, 7, 1023, 4096, 65536 + 3, 300001]
+    esize = dtype.itemsize
+
+    def make(scale):
+        out = []
+        for i, size in enumerate(sizes):
+            flat = torch.empty(size + 8, dtype=dtype, device=device)
+            t = flat[(i % 3):(i % 3) + size]  # some views start off a 16-byte boundary
+            t.copy_((scale * torch.randn(size, generator=gen)).to(dtype).to(device))
+            out.append(t)
+        return out
+
+    def sums():
+        out = []
+        for i, size in enumerate(sizes):
+            bits = torch.randint(0, 2 ** (8 * esize) - 1, (size,), generator=gen, dtype=torch.int64)
+            raw = bits.to(torch.int32 if esize == 4 else torch.int16)
+            flat = torch.empty(size + 8, dtype=dtype, device=device)
+            t = flat[(i % 3):(i % 3) + size]
+            t.copy_(raw.view(dtype).to(device))
+            out.append(t)
+        return out
+
+    for sgd in (ops.OuterSGD(lr=0.7, momentum=0.9, nesterov=True),
+                ops.OuterSGD(lr=0.1, momentum=0.5, dampening=0.1, weight_decay=0.01, nesterov=False),
+                ops.OuterSGD(lr=0.3)):
+        for first in (True, False):
+            g = sums()
+            b1, m1 = make(0.02), (make(1e-3) if sgd.momentum else None)
+            b2 = [t.clone() for t in b1]
+            m2 = [t.clone() for t in m1] if m1 is not None else None
+            # the same misalignment on both sides: clone() re-aligns, so carve again
+            def like(ts):
+                out = []
+                for i, t in enumerate(ts):
+                    flat = torch.empty(t.numel() + 8, dtype=dtype, device=device)
+                    v = flat[(i % 3):(i % 3) + t.numel()]
+                    v.copy_(t)
+                    out.append(v)
+                return out
+            b2, m2 = like(b2), (like(m2) if m2 is not None else None)
+            p1, p2 = like(b1), like(b1)
+            g_avg = like(g)
+            for t in g_avg:
+                ops.reduce_avg_(t, [t], 1, n)            # the pass Manager.allreduce makes
+            ops.mt_outer_sgd(p1, b1, m1, g_avg, sgd, first)
+            g_before = [t.clone() for t in g]
+            ops.mt_outer_sgd(p2, b2, m2, g, sgd, first, grads_are_sums_of=n)
+            for i in range(len(sizes)):
+                assert_bits_equal(g[i], g_before[i], f"sum buffer {i} is only read")
+                assert_bits_equal_up_to_nan_payload(p2[i], p1[i], f"params {i} n={n} first={first}")
+                assert_bits_equal_up_to_nan_payload(b2[i], b1[i], f"backup {i}")
+                if m1 is not None:
+                    assert_bits_equal_up_to_nan_payload(m2[i], m1[i], f"momentum {i}")
+
+
 def test_diloco_no_commit_leaves_state(device):
     """Phase 1 only (should_commit() false): params == backup, backup and momentum untouched."""
     wl = _mlp_workload(2)

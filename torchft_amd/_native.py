@@ -18,7 +18,7 @@ import torch  # noqa: F401  (must precede loading the library, see module docstr
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtorchft_amd.so"
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 MAX_REPLICAS = 8
 MIN_CHUNK_ELEMS = 8192
 MIN_CHUNK_BYTES = 16384  # tft_mt_copy_bytes counts bytes
@@ -85,6 +85,7 @@ SIGNATURES = {
         [POINTER(MtTable), c_uint32, c_uint32, c_uint32, c_int, c_int, c_void_p],
     ),
     "tft_mt_outer_sgd": (c_int, [POINTER(MtTable), c_int, POINTER(SgdParams), c_void_p]),
+    "tft_mt_outer_sgd_of_sum": (c_int, [POINTER(MtTable), c_uint32, c_int, POINTER(SgdParams), c_void_p]),
     "tft_mt_copy_bytes": (c_int, [POINTER(MtTable), c_void_p]),
     "tft_probe_rw_pair": (c_int, [c_void_p, c_void_p, c_uint64, c_void_p]),
 }

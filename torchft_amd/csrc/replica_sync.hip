@@ -603,24 +603,38 @@ struct PseudogradOp {
 };
 
 // columns: [p, b, buf, g]
+// With `divide` set, g holds the SUM of the replicas' pseudo-gradients as a collective left it
+// and is divided by num_participants here, in registers, instead of by a pass of its own
+// over the buffer.  The quotient is rounded to the storage type before it is used
+// (`storage`: 0 fp32, 1 bf16, 2 fp16), as it would have been when that pass stored it.
 struct OuterSgdOp {
   static constexpr int NCOL = 4;
   static constexpr bool kHasFast = true;
   static constexpr bool kStoreSc1 = true;
   SgdCoef k;
+  Divisor d;
+  uint32_t divide;
+  uint32_t storage;
   __device__ inline bool uses_buf() const { return k.momentum != 0.0f; }
   __device__ inline uint32_t rmask() const {
     return 8u | 2u | ((uses_buf() && !k.first_step) ? 4u : 0u);
   }
   __device__ inline uint32_t wmask() const { return 3u | (uses_buf() ? 4u : 0u); }
+  __device__ inline float grad(float g) const {
+    if (!divide) return g;
+    g = d.inv != 0.0f ? __fmul_rn(g, d.inv) : __fdiv_rn(g, d.n);
+    if (storage == 1u) return BF16::widen1(BF16::narrow1(g));
+    if (storage == 2u) return F16::widen1(F16::narrow1(g));
+    return g;
+  }
   __device__ inline void apply(float (&v)[NCOL]) const {
-    const float p = sgd_update(k, v[3], v[1], v[2]);
+    const float p = sgd_update(k, grad(v[3]), v[1], v[2]);
     v[0] = p;
     v[1] = p;
   }
   __device__ inline bool fast() const { return sgd_is_common(k); }
   __device__ inline void apply_fast(float (&v)[NCOL]) const {
-    const float p = sgd_update_common(k, v[3], v[1], v[2]);
+    const float p = sgd_update_common(k, grad(v[3]), v[1], v[2]);
     v[0] = p;
     v[1] = p;
   }
@@ -1174,18 +1188,33 @@ int tft_mt_pseudograd_avg(const tft_mt_table* table, uint32_t n_replicas,
   return rc;
 }
 
-int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd,
-                     void* stream) {
-  static const char* what = "tft_mt_outer_sgd";
+// grad_divisor 0: g is the averaged pseudo-gradient; otherwise g is a sum still to be divided
+static int outer_sgd(const char* what, const tft_mt_table* table, uint32_t grad_divisor, int dtype,
+                     const tft_sgd_params* sgd, void* stream) {
   if (int rc = check_dtype(what, dtype)) return rc;
   if (int rc = check_sgd(what, sgd)) return rc;
   if (int rc = check_table(what, table, 4)) return rc < 0 ? rc : TFT_OK;
-  const OuterSgdOp op{make_coef(sgd)};
+  const uint32_t storage = dtype == TFT_BF16 ? 1u : dtype == TFT_F16 ? 2u : 0u;
+  const OuterSgdOp op{make_coef(sgd), make_divisor(grad_divisor ? grad_divisor : 1u),
+                      grad_divisor ? 1u : 0u, storage};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Shape shape = pick_shape(kFamOuterSgd, table_elems(table) * esize_of(dtype) * 6);
   int rc = TFT_OK;
   TFT_DISPATCH_DTYPE(rc, launch_table, OuterSgdOp, dtype, what, table, op, shape, s);
   return rc;
+}
+
+int tft_mt_outer_sgd(const tft_mt_table* table, int dtype, const tft_sgd_params* sgd,
+                     void* stream) {
+  return outer_sgd("tft_mt_outer_sgd", table, 0, dtype, sgd, stream);
+}
+
+int tft_mt_outer_sgd_of_sum(const tft_mt_table* table, uint32_t num_participants, int dtype,
+                            const tft_sgd_params* sgd, void* stream) {
+  static const char* what = "tft_mt_outer_sgd_of_sum";
+  if (num_participants == 0)
+    return fail(TFT_ERR_INVALID_ARGUMENT, "%s: num_participants must be at least 1", what);
+  return outer_sgd(what, table, num_participants, dtype, sgd, stream);
 }
 
 int tft_mt_diloco_outer_noalloc(const void* const* ptrs, const uint64_t* numel, uint32_t n_tensors,

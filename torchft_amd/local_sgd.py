@@ -437,7 +437,8 @@ class LocalSGD:
                 return
             self._manager.allreduce_tensors(params).wait()
         elif _is_native_manager(self._manager) and self._on_one_gpu(params):
-            self._average_bucketized(params)  # wherever the backup is kept
+            self._sync_bucketized(params, backups)  # wherever the backup is kept
+            return
         else:
             self._average()
         if self._manager.should_commit():
@@ -492,15 +493,40 @@ class LocalSGD:
         self._restore_parameters()
         return False
 
-    def _average_bucketized(self, params: List[torch.Tensor]) -> None:
-        """Flatten (one launch), ONE ``manager.allreduce`` per dtype, unflatten (one launch)."""
+    def _sync_bucketized(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> None:
+        """Through an ordinary process group: flatten (one launch), ONE collective per dtype
+        that leaves the SUM in the flat buffer, and then, if the step is committed, ONE
+        launch that divides by the number of participants and writes the average to the
+        parameters and to the backup (what the reference does in four passes: divide,
+        copy back, save; torchft/manager.py:287, torchft/local_sgd.py:121-125).  A step that
+        is not committed only restores the parameters."""
+        manager = self._manager
         flats, views = self._flat_like("weights", params)
         self._tables["flatten"] = ops.mt_copy(views, params, table=self._tables.get("flatten"))
-        works = [self._manager.allreduce(flat) for flat in flats.values()]
+        works = [manager.allreduce(flat, divide=False) for flat in flats.values()]
         for work in works:
             work.wait()
-        if self._manager.errored() is None:
-            self._tables["unflatten"] = ops.mt_copy(params, views, table=self._tables.get("unflatten"))
+        if not manager.should_commit():
+            self._restore_parameters()
+            return
+        hb = self._host_backup
+        packed = hb is not None and hb.owns(backups)
+        if self._together(params, backups):
+            outs = [params, backups]
+        elif packed:
+            outs = [params, hb.reserve()]  # the backup's device-side staging buffer
+        else:
+            outs = [params]               # a backup kept elsewhere: saved below, tensor by tensor
+        for idx in ops.dtype_groups(params):
+            key = f"unflatten/{params[idx[0]].dtype}"
+            self._tables[key] = ops.mt_reduce_avg(
+                [[col[i] for i in idx] for col in outs], [[views[i] for i in idx]],
+                1, manager.num_participants(), table=self._tables.get(key),
+            )
+        if packed:
+            hb.publish()
+        elif len(outs) == 1:
+            self._save_parameters()
 
     def _average(self) -> None:
         works = []
@@ -724,10 +750,13 @@ class DiLoCo(LocalSGD):
         backups: List[torch.Tensor],
         grads: List[torch.Tensor],
         plan: Optional[List[Tuple[List[int], ops.OuterSGD, bool]]],
+        grads_are_sums_of: Optional[int] = None,
     ) -> None:
         """Committed: apply the outer optimizer to the restored parameters and refresh the
-        backup (torchft/local_sgd.py:221-224)."""
+        backup (torchft/local_sgd.py:221-224).  ``grads_are_sums_of=n`` (fusable SGD only): the
+        gradient buffers hold sums over n participants, divided inside the launch."""
         if plan is None:
+            assert grads_are_sums_of is None
             self._outer_optimizer.step()
             self._save_parameters()
             return
@@ -742,6 +771,7 @@ class DiLoCo(LocalSGD):
                 sgd,
                 first,
                 table=self._tables.get(key),
+                grads_are_sums_of=grads_are_sums_of,
             )
             if first and bufs is not None:
                 self._attach_momentum(idx, bufs)
@@ -802,6 +832,7 @@ class DiLoCo(LocalSGD):
         # committed.  Any other optimizer gets its restore first, as in the reference.
         restore_first = plan is None
         restored = False
+        sums_of: Optional[int] = None  # -1: the gradient buffers hold sums over the participants
         if fused:
             # pseudo-gradient, replica sum and divide (and the restore, if it comes first): one launch
             for p, g in zip(live, grads):
@@ -815,7 +846,11 @@ class DiLoCo(LocalSGD):
             restored = restore_first
             for p, g in zip(live, grads):
                 p.grad = g
-            works = [self._manager.allreduce(flat) for flat in self._flat_like("grads", params)[0].values()]
+            # with a fusable SGD the collective leaves the SUM in the buffer and the outer
+            # step divides on the way in (no pass of its own over the buffer for the division)
+            sums_of = -1 if plan is not None else None
+            works = [self._manager.allreduce(flat, divide=plan is None)
+                     for flat in self._flat_like("grads", params)[0].values()]
             for work in works:
                 work.wait()
         else:
@@ -830,7 +865,9 @@ class DiLoCo(LocalSGD):
 
         committed = self._manager.should_commit()
         if committed:
-            self._outer_step(params, backups, grads, plan)
+            if sums_of is not None:
+                sums_of = self._manager.num_participants()
+            self._outer_step(params, backups, grads, plan, grads_are_sums_of=sums_of)
         elif not restored:
             self._restore_from(params, backups)
         self._outer_optimizer.zero_grad()

@@ -445,9 +445,13 @@ class Manager(Generic[T]):
         return decision
 
     # --------------------------------------------------------------- allreduce
-    def allreduce(self, tensor: torch.Tensor) -> torch.futures.Future:
+    def allreduce(self, tensor: torch.Tensor, *, divide: bool = True) -> torch.futures.Future:
         """In place: zero if this replica does not participate, SUM over the replicas,
         divide by ``num_participants()``; the future resolves to ``tensor`` itself.
+
+        ``divide=False`` (not in the reference) leaves the sum in ``tensor``: for callers
+        whose next kernel reads the buffer anyway and divides on the way in (the bucketised
+        LocalSGD / DiLoCo sync), which saves a pass over the buffer.
 
         Never raises: a failure is latched (``errored()``), the future still
         completes with the (possibly corrupt) tensor and every later call is a no-op
@@ -463,7 +467,7 @@ class Manager(Generic[T]):
             ops.check_tensor(tensor, "Manager.allreduce")
             if hasattr(self._pg, "allreduce_avg"):
                 work = self._pg.allreduce_avg(
-                    [tensor], self.is_participating(), self.num_participants()
+                    [tensor], self.is_participating(), self.num_participants() if divide else 1
                 )
                 fut = work.get_future().then(lambda f: (f.value(), tensor)[1])
             else:
@@ -473,7 +477,8 @@ class Manager(Generic[T]):
 
                 def normalize(f: torch.futures.Future) -> torch.Tensor:
                     f.value()  # surfaces a failed collective
-                    ops.reduce_avg_(tensor, [tensor], 1, self.num_participants())
+                    if divide:
+                        ops.reduce_avg_(tensor, [tensor], 1, self.num_participants())
                     return tensor
 
                 fut = work.get_future().then(normalize)

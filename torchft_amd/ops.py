@@ -212,16 +212,28 @@ def mt_outer_sgd(
     sgd: OuterSGD,
     first_step: bool,
     table: Optional[TensorTable] = None,
+    grads_are_sums_of: Optional[int] = None,
 ) -> TensorTable:
-    """SGD update from backups with grads; writes params, backups (and momentum buffers)."""
+    """SGD update from backups with grads; writes params, backups (and momentum buffers).
+    ``grads_are_sums_of=n``: ``grads`` holds the sum a collective left in it, and every
+    element is divided by n (rounded to the storage dtype) on the way into the update -
+    the division ``Manager.allreduce`` otherwise does in a pass of its own."""
     if sgd.momentum != 0.0 and bufs is None:
         raise ValueError("momentum != 0 needs momentum buffers")
     cols = [params, backups, bufs if bufs is not None else backups, grads]
     if table is None or not table.matches(cols):
         table = TensorTable(cols, what="mt_outer_sgd")
-    _launch(
-        table, "tft_mt_outer_sgd", table.dtype_code, ctypes.byref(sgd.to_struct(first_step))
-    )
+    if grads_are_sums_of is None:
+        _launch(
+            table, "tft_mt_outer_sgd", table.dtype_code, ctypes.byref(sgd.to_struct(first_step))
+        )
+    else:
+        if grads_are_sums_of < 1:
+            raise ValueError("grads_are_sums_of must be at least 1")
+        _launch(
+            table, "tft_mt_outer_sgd_of_sum", int(grads_are_sums_of), table.dtype_code,
+            ctypes.byref(sgd.to_struct(first_step)),
+        )
     return table
 
 
