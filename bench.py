@@ -40,6 +40,7 @@ HEADLINE_METRIC = "outer-sync params/sec + achieved HBM GB/s (% peak), Llama-3-8
 WORKLOADS = ["diloco_llama3_8b", "diloco_gpt2_small", "ddp_buckets_llama3_8b",
              "checkpoint_llama3_8b", "localsgd_llama3_8b", "diloco_llama3_8b_api",
              "diloco_two_phase_llama3_8b", "placement_llama3_8b_slice", "host_backup_llama3_8b",
+             "diloco_bucketized_llama3_8b", "localsgd_bucketized_llama3_8b",
              "ddp_buckets_llama3_8b_two_streams", "ddp_whole_model_llama3_8b", "localsgd_llama3_8b_api",
              "ddp_hook_llama3_8b", "diloco_gpt2_small_api"]
 
@@ -575,6 +576,101 @@ def bench_localsgd_api(args) -> Dict[str, object]:
                      "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2})
     out["roofline"] = roofline(n_params * 16, kernel_ms, "mt_stream_kernel<F32, ReduceAvgOp<2, 2>>")
     out["roofline"]["note"] = "kernel_ms_per_step here spans the whole sync() on the stream, host gaps included"
+    return out
+
+
+def bench_bucketized_api(args, kind: str) -> Dict[str, object]:
+    """What one GPU does per sync when the replicas live on different GPUs: ``DiLoCo.sync()`` /
+    ``LocalSGD.sync()`` over an ORDINARY process group (one collective per dtype on a flat
+    buffer).  The collective itself is not this build's (one GPU): the group here returns at
+    once, as if the peer had contributed zeros, so the timed sync is the local work around it.
+    DiLoCo: pseudo-gradients into the flat buffer (12 B/param), the collective leaves the sum,
+    the outer SGD divides on the way in and writes parameters, backup and momentum (24 B).
+    LocalSGD: flatten (8 B), collective, then one launch that divides and writes parameters and
+    backup (12 B)."""
+    from torch import nn
+
+    from oracle import replica_sync as O  # the checker of the first sync's output, nothing else
+    from torchft_amd import DiLoCo, LocalSGD, Manager, ProcessGroup, StaticQuorum, workloads
+    from torchft_amd.process_group import _DummyWork
+
+    class SumWithAZeroPeer(ProcessGroup):
+        def __init__(self) -> None:
+            super().__init__(0, 2)
+            self.calls = 0
+
+        def configure(self, store_addr: str, rank: int, world_size: int) -> None:
+            pass
+
+        def allreduce(self, tensors, opts):
+            self.calls += 1
+            return _DummyWork(tensors)
+
+        def size(self) -> int:
+            return 2
+
+        def getBackendName(self) -> str:
+            return "sum-with-a-zero-peer"
+
+    dev = torch.device("cuda", 0)
+    shapes = workloads.llama3_8b_shapes()
+
+    class Bag(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.ps = nn.ParameterList(
+                [nn.Parameter(t) for t in workloads.normal_tensors(shapes, 0.02, 0, dev)])
+
+    model = Bag()
+    pg = SumWithAZeroPeer()
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner = torch.optim.SGD(model.parameters(), lr=0.1)
+    n_params = sum(p.numel() for p in model.parameters())
+    check = [2, 146]
+    params = [p.data for p in model.parameters()]
+    if kind == "diloco":
+        outer = torch.optim.SGD(model.parameters(), lr=LR, momentum=MOMENTUM, nesterov=True)
+        ctx = DiLoCo(manager, model, inner, outer, sync_every=10 ** 9)
+        per_param = 36
+    else:
+        ctx = LocalSGD(manager, model, inner, sync_every=10 ** 9)
+        per_param = 20
+    with ctx:
+        backups = list(ctx._backup_parameters.values())
+        # the first sync, checked: a drift of the parameters against the backup
+        for i in check:
+            params[i].add_(1e-3)
+        local = [params[i].cpu() for i in check]
+        before = [backups[i].cpu() for i in check]
+        ctx.sync()
+        torch.cuda.synchronize()
+        if kind == "diloco":
+            want = O.diloco_perform_sync([local, before], before, None, [True, True], 2, True,
+                                         lr=LR, momentum=MOMENTUM, nesterov=True)
+        else:
+            zeros = [torch.zeros_like(t) for t in local]
+            want = O.localsgd_perform_sync([local, zeros], before, [True, True], 2, True)
+        for k, i in enumerate(check):
+            if not (torch.equal(params[i].cpu(), want["params"][k]) and torch.equal(backups[i].cpu(), want["backup"][k])):
+                raise RuntimeError(f"output check failed: tensor {i} differs from the CPU checker's result")
+        calls = pg.calls
+        wall_ms, kernel_ms = Timed(args.steps, args.warmup).run(ctx.sync)
+        per_sync = (pg.calls - calls) / (args.steps + args.warmup)
+    manager.shutdown(wait=False)
+    name = "DiLoCo" if kind == "diloco" else "LocalSGD"
+    out = base_line(args, f"{name} sync over an ordinary process group, local work, params/sec, Llama-3-8B",
+                    n_params / (wall_ms * 1e-3), "params/s", wall_ms, "f32",
+                    {"workload": f"{name}.sync() on a module with the 291 Llama-3-8B fp32 parameters over an ordinary "
+                                 "process group (bucketised: one collective per sync on a flat buffer; the "
+                                 "collective returns at once, the peer contributing zeros), 2 replicas",
+                     "n_tensors": len(shapes), "n_params": n_params, "n_replicas": 2,
+                     "collectives_per_sync": per_sync,
+                     "output_check": f"first sync: parameters and backup of tensors {check} equal the CPU checker's bit for bit"})
+    out["roofline"] = roofline(n_params * per_param, kernel_ms,
+                               "PseudogradOp<1> + OuterSgdOp" if kind == "diloco" else "mt_copy_kernel + ReduceAvgOp<2, 1>")
+    out["roofline"]["launches_per_step"] = 2
+    out["roofline"]["note"] = "kernel_ms_per_step spans the whole sync() on the stream: two launches and the host between them"
     return out
 
 
@@ -1561,6 +1657,10 @@ def main() -> int:
         out = bench_diloco_two_phase(args)
     elif args.workload == "localsgd_llama3_8b_api":
         out = bench_localsgd_api(args)
+    elif args.workload == "diloco_bucketized_llama3_8b":
+        out = bench_bucketized_api(args, "diloco")
+    elif args.workload == "localsgd_bucketized_llama3_8b":
+        out = bench_bucketized_api(args, "localsgd")
     elif args.workload == "placement_llama3_8b_slice":
         out = bench_placement(args)
     elif args.workload == "host_backup_llama3_8b":
