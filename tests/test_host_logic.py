@@ -1002,6 +1002,45 @@ def test_diloco_bucketized_failed_collective_discards_the_step(cpu_ops, outer_ki
     manager.shutdown(wait=False)
 
 
+@pytest.mark.parametrize("outer_kind", ["sgd_nesterov", "adam"])
+def test_diloco_bucketized_matches_the_reference_loop(cpu_ops, outer_kind):
+    """Through an ordinary process group whose peer contributes what this replica does (SUM
+    doubles, the average is the replica's own pseudo-gradient again): the wrapper leaves the
+    model where the reference's loop over one replica would, with the outer SGD that divides
+    the sum on the way in and with an optimizer that steps on the averaged ``p.grad``."""
+    torch.manual_seed(3)
+    model = SimpleModel()
+    twin = SimpleModel()
+    twin.load_state_dict(model.state_dict())
+
+    def make_outer(m):
+        if outer_kind == "adam":
+            return optim.Adam(m.parameters(), lr=1e-2)
+        return optim.SGD(m.parameters(), lr=0.7, momentum=0.9, nesterov=True)
+
+    pg = _DoublingPG()
+    manager = Manager(pg=pg, load_state_dict=None, state_dict=None, min_replica_size=2, use_async_quorum=False,
+                      quorum_client=StaticQuorum(0, 2))
+    inner, outer = optim.SGD(model.parameters(), lr=0.1), make_outer(model)
+    twin_inner, twin_outer = optim.SGD(twin.parameters(), lr=0.1), make_outer(twin)
+    twin_backup = [p.data.clone() for p in twin.parameters()]
+    gloo = O.make_gloo_world1()
+    with DiLoCo(manager, model, inner, outer, sync_every=2):
+        for step in range(6):
+            x = torch.rand(2, 3)
+            for m, o in ((model, inner), (twin, twin_inner)):
+                o.zero_grad()
+                m(x).mean().backward()
+                o.step()
+            if step % 2 == 1:
+                O.diloco_reference_loop_(gloo, list(twin.parameters()), twin_backup, [], twin_outer, 1)
+            for a, b in zip(model.parameters(), twin.parameters()):
+                assert_bits_equal(a.data, b.data, f"step {step}")
+    assert len(pg.calls) == 3  # one collective per sync
+    assert (cpu_ops.calls.count("mt_outer_sgd") == 3) == (outer_kind == "sgd_nesterov")
+    manager.shutdown(wait=False)
+
+
 def test_local_sgd_bucketized_one_collective_per_sync(cpu_ops):
     torch.manual_seed(0)
     model = SimpleModel()
