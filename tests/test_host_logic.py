@@ -1256,6 +1256,52 @@ def test_local_sgd_fused_applies_recovered_state_with_asynchronous_quorum(cpu_op
     manager.shutdown(wait=False)
 
 
+@pytest.mark.parametrize("group", ["local_replicas", "ordinary"])
+def test_local_sgd_ends_with_the_recovered_state_when_the_vote_loads_it(cpu_ops, group):
+    """A healing replica under an asynchronous quorum whose ``load_state_dict`` really loads the
+    model: the reference averages first and the vote then loads the recovered state over it
+    (torchft/local_sgd.py:151-158, torchft/manager.py:572-575), so the sync ends with the
+    recovered parameters, and the backup equals them."""
+    import time
+
+    torch.manual_seed(4)
+    model = SimpleModel()
+    peers, lookup = _replica_world(model, 2)
+    recovered = {k: torch.full_like(v, 0.125) for k, v in model.state_dict().items()}
+
+    class HealingQuorum(QuorumClient):
+        def quorum(self, rank, step, checkpoint_metadata, shrink_only, timeout):
+            time.sleep(0.1)
+            return QuorumResult(quorum_id=7, replica_rank=0, replica_world_size=2,
+                                recover_src_manager_address="peer", recover_src_rank=1,
+                                max_step=5, max_rank=None, max_world_size=1, heal=True)
+
+        def should_commit(self, rank, step, should_commit, timeout):
+            return should_commit
+
+        def checkpoint_metadata(self, address, rank, timeout):
+            return "meta"
+
+    transport = MagicMock()
+    transport.metadata.return_value = ""
+    transport.recv_checkpoint.return_value = {"user": recovered, "torchft": {"step": 5, "batches_committed": 10}}
+    pg = (ProcessGroupLocalReplicas(rank=0, world_size=2, peer_lookup=lookup) if group == "local_replicas"
+          else _DoublingPG())
+    manager = Manager(pg=pg, load_state_dict=model.load_state_dict, state_dict=model.state_dict, min_replica_size=1,
+                      use_async_quorum=True, quorum_client=HealingQuorum(), checkpoint_transport=transport)
+    optimizer = optim.SGD(model.parameters(), lr=0.1)
+    with LocalSGD(manager, model, optimizer, sync_every=1) as lsgd:
+        with torch.no_grad():
+            for p in model.parameters():
+                p.grad = torch.zeros_like(p)
+        optimizer.step()
+        assert manager.current_step() == 6
+        for (name, p), b in zip(model.named_parameters(), lsgd._backup_parameters.values()):
+            assert_bits_equal(p.data, recovered[name], name)
+            assert_bits_equal(b, recovered[name], f"backup {name}")
+    manager.shutdown(wait=False)
+
+
 # ---------------------------------------------------------------------------
 # What a wrapper keeps between syncs, and what makes it look again
 # ---------------------------------------------------------------------------

@@ -420,6 +420,24 @@ class LocalSGD:
         """Average, then keep the result (commit) or roll back (torchft/local_sgd.py:151-162)."""
         _, params, backups = self._named()
         hb = self._host_backup
+        if _is_native_manager(self._manager):
+            self._manager.wait_quorum()
+            if self._manager.applies_recovered_state_in_vote():
+                # Healing under an asynchronous quorum: the vote loads the recovered state
+                # dict over whatever the reduction has written (torchft/manager.py:572-575).
+                # Only the reference's own order of steps - average into the parameters, vote,
+                # save or restore - ends where the reference ends, so this (rare) sync takes it.
+                if self._fused(params, backups):
+                    self._manager.allreduce_tensors(params).wait()
+                elif self._on_one_gpu(params):
+                    self._average_bucketized(params)
+                else:
+                    self._average()
+                if self._manager.should_commit():
+                    self._save_parameters()
+                else:
+                    self._restore_parameters()
+                return
         if (
             hb is not None
             and hb.owns(backups)
@@ -492,6 +510,17 @@ class LocalSGD:
             return True
         self._restore_parameters()
         return False
+
+    def _average_bucketized(self, params: List[torch.Tensor]) -> None:
+        """Flatten (one launch), ONE ``manager.allreduce`` per dtype, unflatten (one launch): the
+        average is in the parameters before the vote, as in the reference."""
+        flats, views = self._flat_like("weights", params)
+        self._tables["flatten"] = ops.mt_copy(views, params, table=self._tables.get("flatten"))
+        works = [self._manager.allreduce(flat) for flat in flats.values()]
+        for work in works:
+            work.wait()
+        if self._manager.errored() is None:
+            self._tables["unflatten"] = ops.mt_copy(params, views, table=self._tables.get("unflatten"))
 
     def _sync_bucketized(self, params: List[torch.Tensor], backups: List[torch.Tensor]) -> None:
         """Through an ordinary process group: flatten (one launch), ONE collective per dtype

@@ -344,6 +344,12 @@ class Manager(Generic[T]):
         assert self._quorum_future is not None, "must call start_quorum before wait_quorum"
         self._quorum_future.result()
 
+    def applies_recovered_state_in_vote(self) -> bool:
+        """After ``wait_quorum()``: True for a replica that is healing under an asynchronous
+        quorum.  Its recovered state dict is loaded by ``should_commit()``
+        (torchft/manager.py:572-575), over whatever a reduction has written before."""
+        return self._healing
+
     def _async_quorum(self, allow_heal: bool, shrink_only: bool, quorum_timeout: timedelta) -> None:
         metadata = self._checkpoint_transport.metadata() if self._checkpoint_transport else ""
         q = self._client.quorum(
