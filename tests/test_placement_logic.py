@@ -386,3 +386,27 @@ def test_a_model_scattered_over_the_groups_is_measured_tensor_by_tensor(small_co
     assert copies is not None
     for t, c in zip(like, copies[0]):
         assert dev.group_at(c) != dev.group_at(t)
+
+
+def test_a_model_without_a_tensor_long_enough_to_time_is_left_alone(monkeypatch):
+    """300 MiB of parameters in tensors of 1 MiB: nothing can tell which group they lie in, so
+    no search is started (and no device memory is taken for one)."""
+    monkeypatch.setattr(H, "enabled", lambda: True)
+    started = []
+    monkeypatch.setattr(H, "_locked_search", lambda *a, **k: started.append(1))
+
+    class OnGpu:  # what allocate_apart reads of a tensor
+        device = torch.device("cuda", 0)
+
+        def __init__(self, n):
+            self.n = n
+
+        def numel(self):
+            return self.n
+
+        def element_size(self):
+            return 4
+
+    assert H.allocate_apart([OnGpu(MiB // 4)] * 300, 2) is None and not started
+    H.allocate_apart([OnGpu(MiB // 4)] * 300 + [OnGpu(64 * MiB)], 2)
+    assert started == [1]

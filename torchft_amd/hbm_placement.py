@@ -49,8 +49,8 @@ wrapper takes its first backup of them).
 
 Nothing here affects results: a wrong or impossible placement only costs
 bandwidth.  ``TORCHFT_AMD_HBM_PLACEMENT=0`` switches the probing off, and it is
-skipped by itself for models too small to matter or when the timings show no
-group structure (other GPUs).
+skipped by itself for models too small to matter, for models without a tensor
+long enough to time, or when the timings show no group structure (other GPUs).
 """
 
 from __future__ import annotations
@@ -518,6 +518,12 @@ def allocate_apart(
         return None
     sizes = [t.numel() * t.element_size() for t in like]
     if sum(sizes) < MIN_MODEL_BYTES:
+        return None
+    if max(sizes) < MIN_PROBE_BYTES:
+        # no tensor long enough to time: which group the model lies in cannot be told, so
+        # there is nothing to place the copies away from
+        logger.info("hbm placement: no tensor of %d MiB or more in the model; default allocation",
+                    MIN_PROBE_BYTES >> 20)
         return None
     return _locked_search(device_state(device), like, sizes, n_copies, device)
 
